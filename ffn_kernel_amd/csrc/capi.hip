@@ -1,0 +1,333 @@
+// C ABI of libffnk (declared in include/ffnk.h): argument checks, workspace carving, path
+// selection and kernel sequencing.  Nothing here allocates, frees or synchronises.
+#include "../../include/ffnk.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.hpp"
+#include "launch.hpp"
+#include "tile_table.hpp"
+
+using namespace ffnk;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+  return (int)e;
+}
+
+#define FFNK_HIP(expr, what)                       \
+  do {                                             \
+    hipError_t e__ = (expr);                       \
+    if (e__ != hipSuccess) return hip_fail(e__, what); \
+  } while (0)
+
+constexpr int64_t kMaxRows = (int64_t)1 << 30;
+constexpr int64_t kMaxCols = (int64_t)1 << 24;
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1) == 0; }
+
+int check_extents(int64_t M, int64_t K, int64_t N) {
+  if (M < 0 || K < 0 || N < 0) return fail(FFNK_E_SHAPE, "negative extent M=%lld K=%lld N=%lld", (long long)M, (long long)K, (long long)N);
+  if (M > kMaxRows) return fail(FFNK_E_SHAPE, "M=%lld exceeds %lld rows", (long long)M, (long long)kMaxRows);
+  if (K > kMaxCols || N > kMaxCols) return fail(FFNK_E_SHAPE, "K=%lld or N=%lld exceeds %lld", (long long)K, (long long)N, (long long)kMaxCols);
+  return FFNK_OK;
+}
+
+// Workspace regions.
+struct RouteWs {
+  int32_t* perm;
+  int32_t* counts;
+  size_t bytes;
+};
+size_t route_ws_bytes(int64_t M) { return ws_align((size_t)M * 4) + ws_align(8); }
+RouteWs carve_route(uint8_t* ws, int64_t M) {
+  RouteWs r;
+  r.perm = reinterpret_cast<int32_t*>(ws);
+  r.counts = reinterpret_cast<int32_t*>(ws + ws_align((size_t)M * 4));
+  r.bytes = route_ws_bytes(M);
+  return r;
+}
+
+int64_t padded_rows(int64_t M) { return round_up64(M, 64) + 64; }  // >= pad64(nv) + pad64(M - nv)
+
+struct BwdPlan {
+  bool dw_k_contig;  // dW memory is [N, K] (k contiguous): R = N, Cc = K
+  int64_t R, Cc;
+  TileChoice tc;
+  int64_t ldt;       // row stride of the transposed operands
+  size_t off_wt, off_gt, off_xt, off_p, total;
+};
+BwdPlan plan_bwd(int64_t M, int64_t K, int64_t N, bool dw_k_contig) {
+  BwdPlan p;
+  p.dw_k_contig = dw_k_contig;
+  p.R = dw_k_contig ? N : K;
+  p.Cc = dw_k_contig ? K : N;
+  p.tc = pick_splitk_tile(M, p.R, p.Cc);
+  p.ldt = padded_rows(M);
+  size_t o = route_ws_bytes(M);
+  p.off_wt = o; o += 2 * ws_align((size_t)K * N * 2);
+  p.off_gt = o; o += ws_align((size_t)N * p.ldt * 2);
+  p.off_xt = o; o += ws_align((size_t)K * p.ldt * 2);
+  p.off_p = o;  o += ws_align((size_t)2 * p.tc.splits * K * N * 4);
+  p.total = o;
+  return p;
+}
+
+bool use_stream_path(int64_t M) { return false && M <= kStreamMaxM; }
+
+}  // namespace
+
+extern "C" {
+
+int ffnk_version(void) { return FFNK_VERSION; }
+
+const char* ffnk_last_error(void) { return g_err; }
+
+int ffnk_route(const uint8_t* mask, int64_t M, int32_t* perm, int32_t* counts, void* stream) {
+  if (int e = check_extents(M, 0, 0)) return e;
+  if (!counts || (M > 0 && (!mask || !perm))) return fail(FFNK_E_NULL, "ffnk_route: NULL pointer");
+  FFNK_HIP(launch_route(mask, (int)M, perm, counts, (hipStream_t)stream), "route kernel");
+  return FFNK_OK;
+}
+
+size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
+  if (M < 0 || K < 0 || N < 0 || M > kMaxRows || K > kMaxCols || N > kMaxCols) return (size_t)-1;
+  switch (op) {
+    case FFNK_OP_LINEAR_FWD:
+      return route_ws_bytes(M);
+    case FFNK_OP_FFN_FWD:
+      // perm + counts + the [M, h] bf16 intermediate in routed order (N = h).
+      return route_ws_bytes(M) + ws_align((size_t)M * round_up64(N, 8) * 2);
+    case FFNK_OP_LINEAR_BWD: {
+      const BwdPlan a = plan_bwd(M, K, N, true), b = plan_bwd(M, K, N, false);
+      return a.total > b.total ? a.total : b.total;
+    }
+    default:
+      return (size_t)-1;
+  }
+}
+
+int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t* out) {
+  if (!out) return fail(FFNK_E_NULL, "ffnk_tile_config: out is NULL");
+  if (int e = check_extents(M, K, N)) return e;
+  memset(out, 0, sizeof(*out));
+  int tile;
+  bool dual = false;
+  int64_t contraction;
+  int splits = 1;
+  switch (op) {
+    case FFNK_OP_LINEAR_FWD: tile = pick_routed_tile(M, N, false); contraction = K; break;
+    case FFNK_OP_FFN_FWD:
+    case FFNK_OP_FFN_UP: tile = pick_routed_tile(M, N, true); dual = true; contraction = K; break;
+    case FFNK_OP_FFN_DOWN: tile = pick_routed_tile(M, K, false); contraction = N; break;  // out cols = d = K, contraction h = N
+    case FFNK_OP_LINEAR_BWD:
+    case FFNK_OP_BWD_DX: tile = pick_routed_tile(M, K, false); contraction = N; break;
+    case FFNK_OP_BWD_DW: {
+      const TileChoice c = pick_splitk_tile(M, N, K);
+      tile = c.tile; splits = c.splits; contraction = M; break;
+    }
+    default: return fail(FFNK_E_OP, "unknown op %d", op);
+  }
+  const TileGeom gm = tile_geom(tile, dual);
+  const bool stream = (op == FFNK_OP_FFN_FWD || op == FFNK_OP_FFN_UP || op == FFNK_OP_FFN_DOWN) && use_stream_path(M);
+  out->path = stream ? FFNK_PATH_STREAM : FFNK_PATH_MFMA_TILED;
+  out->block_m = gm.block_m;
+  out->block_n = gm.block_n_out;
+  out->block_k = 64;
+  out->waves_m = gm.waves_m;
+  out->waves_n = gm.waves_n;
+  out->lds_stages = 2;
+  out->group_m = 8;
+  out->split_k = splits;
+  out->direct_lds = (contraction % 64 == 0) ? 1 : 0;
+  return FFNK_OK;
+}
+
+int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t* Wv, const uint16_t* Wt,
+                           int64_t w_stride_k, int64_t w_stride_n, const uint8_t* mask, uint16_t* y,
+                           int64_t y_stride_m, int64_t M, int64_t K, int64_t N, void* ws, size_t ws_bytes,
+                           void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (int e = check_extents(M, K, N)) return e;
+  if (M == 0 || N == 0) return FFNK_OK;
+  if (!x && K > 0) return fail(FFNK_E_NULL, "x is NULL");
+  if ((!Wv || !Wt) && K > 0) return fail(FFNK_E_NULL, "weight pointer is NULL");
+  if (!mask || !y) return fail(FFNK_E_NULL, "mask or y is NULL");
+  if (!aligned2(x) || !aligned2(Wv) || !aligned2(Wt) || !aligned2(y)) return fail(FFNK_E_ALIGN, "bf16 pointer not 2-byte aligned");
+  if (y_stride_m < N) return fail(FFNK_E_STRIDE, "y_stride_m=%lld < N=%lld", (long long)y_stride_m, (long long)N);
+
+  const bool fast = K > 0 && K % 8 == 0 && x_stride_m % 8 == 0 && x_stride_m >= K && aligned16(x) &&
+                    w_stride_k == 1 && w_stride_n % 8 == 0 && w_stride_n >= K && aligned16(Wv) && aligned16(Wt);
+  if (!fast) {
+    GenericLinearArgs a;
+    a.x = x; a.sxm = x_stride_m; a.sxk = 1;
+    a.W[0] = Wv; a.W[1] = Wt; a.swk = w_stride_k; a.swn = w_stride_n;
+    a.mask = mask; a.y = y; a.sym = y_stride_m; a.syn = 1;
+    a.M = (int)M; a.K = (int)K; a.N = (int)N;
+    FFNK_HIP(launch_generic_linear(a, stream), "generic linear kernel");
+    return FFNK_OK;
+  }
+  if (ws_bytes < route_ws_bytes(M) || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, route_ws_bytes(M));
+  if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
+  const RouteWs r = carve_route(static_cast<uint8_t*>(ws), M);
+  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+  GemmArgs g;
+  g.A = x; g.lda = x_stride_m;
+  g.B0[0] = Wv; g.B0[1] = Wt; g.B1[0] = g.B1[1] = nullptr; g.ldb = w_stride_n;
+  g.C = y; g.ldc = y_stride_m;
+  g.perm = r.perm; g.counts = r.counts;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  FFNK_HIP(launch_linear_gemm(pick_routed_tile(M, N, false), K % 64 == 0, g, stream), "linear GEMM");
+  return FFNK_OK;
+}
+
+int ffnk_masked_ffn_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, const uint16_t* W3,
+                        const uint16_t* U1, const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n,
+                        const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
+                        const uint8_t* mask, uint16_t* out, int64_t out_stride_m, int64_t M, int64_t d,
+                        int64_t h, void* ws, size_t ws_bytes, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (int e = check_extents(M, d, h)) return e;
+  if (M == 0 || d == 0) return FFNK_OK;
+  if (!x || !mask || !out) return fail(FFNK_E_NULL, "x, mask or out is NULL");
+  if (h > 0 && (!W1 || !W3 || !U1 || !U3 || !W2 || !U2)) return fail(FFNK_E_NULL, "weight pointer is NULL");
+  if (!aligned2(x) || !aligned2(out) || !aligned2(W1) || !aligned2(W3) || !aligned2(U1) || !aligned2(U3) ||
+      !aligned2(W2) || !aligned2(U2))
+    return fail(FFNK_E_ALIGN, "bf16 pointer not 2-byte aligned");
+  if (out_stride_m < d) return fail(FFNK_E_STRIDE, "out_stride_m=%lld < d=%lld", (long long)out_stride_m, (long long)d);
+  const size_t need = ffnk_workspace_bytes(FFNK_OP_FFN_FWD, M, d, h);
+  if (ws_bytes < need || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, need);
+  if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
+
+  uint8_t* wsb = static_cast<uint8_t*>(ws);
+  const RouteWs r = carve_route(wsb, M);
+  uint16_t* H = reinterpret_cast<uint16_t*>(wsb + r.bytes);
+  const int64_t ldh = round_up64(h, 8);
+
+  const bool fast = d % 8 == 0 && h > 0 && h % 8 == 0 && x_stride_m % 8 == 0 && x_stride_m >= d && aligned16(x) &&
+                    up_stride_k == 1 && up_stride_n % 8 == 0 && up_stride_n >= d && down_stride_k == 1 &&
+                    down_stride_n % 8 == 0 && down_stride_n >= h && aligned16(W1) && aligned16(W3) &&
+                    aligned16(U1) && aligned16(U3) && aligned16(W2) && aligned16(U2);
+  if (!fast) {
+    // Token-order intermediate, then the generic routed linear on it.
+    GenericUpArgs u;
+    u.x = x; u.sxm = x_stride_m;
+    u.G[0] = W1; u.G[1] = U1; u.U[0] = W3; u.U[1] = U3; u.swk = up_stride_k; u.swn = up_stride_n;
+    u.mask = mask; u.H = H; u.ldh = ldh;
+    u.M = (int)M; u.K = (int)d; u.N = (int)h;
+    FFNK_HIP(launch_generic_up(u, stream), "generic up kernel");
+    GenericLinearArgs a;
+    a.x = H; a.sxm = ldh; a.sxk = 1;
+    a.W[0] = W2; a.W[1] = U2; a.swk = down_stride_k; a.swn = down_stride_n;
+    a.mask = mask; a.y = out; a.sym = out_stride_m; a.syn = 1;
+    a.M = (int)M; a.K = (int)h; a.N = (int)d;
+    FFNK_HIP(launch_generic_linear(a, stream), "generic down kernel");
+    return FFNK_OK;
+  }
+
+  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+  GemmArgs up;
+  up.A = x; up.lda = x_stride_m;
+  up.B0[0] = W1; up.B0[1] = U1; up.B1[0] = W3; up.B1[1] = U3; up.ldb = up_stride_n;
+  up.C = H; up.ldc = ldh;
+  up.perm = r.perm; up.counts = r.counts;
+  up.M = (int)M; up.N = (int)h; up.K = (int)d;
+  FFNK_HIP(launch_up_gemm(pick_routed_tile(M, h, true), d % 64 == 0, up, stream), "up-projection GEMM");
+  GemmArgs dn;
+  dn.A = H; dn.lda = ldh;
+  dn.B0[0] = W2; dn.B0[1] = U2; dn.B1[0] = dn.B1[1] = nullptr; dn.ldb = down_stride_n;
+  dn.C = out; dn.ldc = out_stride_m;
+  dn.perm = r.perm; dn.counts = r.counts;
+  dn.M = (int)M; dn.N = (int)d; dn.K = (int)h;
+  FFNK_HIP(launch_down_gemm(pick_routed_tile(M, d, false), h % 64 == 0, dn, stream), "down-projection GEMM");
+  return FFNK_OK;
+}
+
+int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,
+                           const uint16_t* Wv, const uint16_t* Wt, int64_t w_stride_k, int64_t w_stride_n,
+                           const uint8_t* mask, uint16_t* dx, int64_t dx_stride_m, uint16_t* dWv, uint16_t* dWt,
+                           int64_t dw_stride_k, int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, void* ws,
+                           size_t ws_bytes, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (int e = check_extents(M, K, N)) return e;
+  if (K == 0) return FFNK_OK;  // dx and dW are empty
+  if (M > 0 && (!mask || !dx || !x)) return fail(FFNK_E_NULL, "mask, x or dx is NULL");
+  if (M > 0 && N > 0 && (!g || !Wv || !Wt)) return fail(FFNK_E_NULL, "g or weight pointer is NULL");
+  if (N > 0 && (!dWv || !dWt)) return fail(FFNK_E_NULL, "dW pointer is NULL");
+  if (!aligned2(g) || !aligned2(x) || !aligned2(Wv) || !aligned2(Wt) || !aligned2(dx) || !aligned2(dWv) || !aligned2(dWt))
+    return fail(FFNK_E_ALIGN, "bf16 pointer not 2-byte aligned");
+  if (dx_stride_m < K) return fail(FFNK_E_STRIDE, "dx_stride_m=%lld < K=%lld", (long long)dx_stride_m, (long long)K);
+
+  const bool fast = M > 0 && N > 0 && K % 8 == 0 && N % 8 == 0 && g_stride_m % 8 == 0 && g_stride_m >= N &&
+                    x_stride_m % 8 == 0 && x_stride_m >= K && aligned16(g) && aligned16(x);
+  if (!fast) {
+    GenericBwdArgs a;
+    a.g = g; a.sgm = g_stride_m; a.x = x; a.sxm = x_stride_m;
+    a.W[0] = Wv; a.W[1] = Wt; a.swk = w_stride_k; a.swn = w_stride_n;
+    a.mask = mask; a.dx = dx; a.sdxm = dx_stride_m;
+    a.dW[0] = dWv; a.dW[1] = dWt; a.sdk = dw_stride_k; a.sdn = dw_stride_n;
+    a.M = (int)M; a.K = (int)K; a.N = (int)N;
+    FFNK_HIP(launch_generic_bwd(a, stream), "generic backward kernels");
+    return FFNK_OK;
+  }
+
+  const BwdPlan p = plan_bwd(M, K, N, dw_stride_k == 1);
+  if (ws_bytes < p.total || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, p.total);
+  if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
+  uint8_t* wsb = static_cast<uint8_t*>(ws);
+  const RouteWs r = carve_route(wsb, M);
+  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+
+  // ---- dx = gather(g) @ W_g^T, contraction over N: needs the weights as [K, N] rows, N contiguous ----
+  const uint16_t* wt[2] = {Wv, Wt};
+  int64_t ldw = w_stride_k;
+  const bool w_direct = w_stride_n == 1 && w_stride_k % 8 == 0 && w_stride_k >= N && aligned16(Wv) && aligned16(Wt);
+  if (!w_direct) {
+    uint16_t* c0 = reinterpret_cast<uint16_t*>(wsb + p.off_wt);
+    uint16_t* c1 = reinterpret_cast<uint16_t*>(wsb + p.off_wt + ws_align((size_t)K * N * 2));
+    FFNK_HIP(launch_strided_copy2d(Wv, w_stride_k, w_stride_n, c0, N, (int)K, (int)N, stream), "weight transpose");
+    FFNK_HIP(launch_strided_copy2d(Wt, w_stride_k, w_stride_n, c1, N, (int)K, (int)N, stream), "weight transpose");
+    wt[0] = c0; wt[1] = c1; ldw = N;
+  }
+  GemmArgs a;
+  a.A = g; a.lda = g_stride_m;
+  a.B0[0] = wt[0]; a.B0[1] = wt[1]; a.B1[0] = a.B1[1] = nullptr; a.ldb = ldw;
+  a.C = dx; a.ldc = dx_stride_m;
+  a.perm = r.perm; a.counts = r.counts;
+  a.M = (int)M; a.N = (int)K; a.K = (int)N;
+  FFNK_HIP(launch_linear_gemm(pick_routed_tile(M, K, false), N % 64 == 0, a, stream), "dx GEMM");
+
+  // ---- dW_g = x_g^T g_g, contraction over the rows of group g ----
+  uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]
+  uint16_t* XT = reinterpret_cast<uint16_t*>(wsb + p.off_xt);  // [K, ldt]
+  float* P = reinterpret_cast<float*>(wsb + p.off_p);
+  FFNK_HIP(launch_gather_transpose(g, g_stride_m, r.perm, r.counts, GT, p.ldt, (int)M, (int)N, stream), "g transpose");
+  FFNK_HIP(launch_gather_transpose(x, x_stride_m, r.perm, r.counts, XT, p.ldt, (int)M, (int)K, stream), "x transpose");
+  SplitKArgs s;
+  s.A = p.dw_k_contig ? GT : XT; s.lda = p.ldt;
+  s.B = p.dw_k_contig ? XT : GT; s.ldb = p.ldt;
+  s.P = P; s.counts = r.counts; s.M = (int)M;
+  s.R = (int)p.R; s.Cc = (int)p.Cc; s.splits = p.tc.splits;
+  FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
+  const int64_t sr = p.dw_k_contig ? dw_stride_n : dw_stride_k;
+  const int64_t sc = p.dw_k_contig ? dw_stride_k : dw_stride_n;
+  FFNK_HIP(launch_splitk_reduce(P, p.tc.splits, (int)p.R, (int)p.Cc, dWv, dWt, sr, sc, stream), "dW reduce");
+  return FFNK_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,34 @@
+// Plain argument blocks of the tiled GEMM kernels (shared by host launch code and device code).
+#pragma once
+#include <stdint.h>
+
+namespace ffnk {
+
+struct GemmArgs {
+  const uint16_t* A;     // [*, K] rows, K contiguous
+  int64_t lda;
+  const uint16_t* B0[2]; // per group (0 = visual, 1 = text): [N, K] rows, K contiguous
+  const uint16_t* B1[2]; // SwiGLU kernels only: second weight (the "up" projection), same shape
+  int64_t ldb;
+  uint16_t* C;           // [*, N] rows
+  int64_t ldc;
+  const int32_t* perm;   // routed position -> token row
+  const int32_t* counts; // counts[0] = visual rows (device memory)
+  int M, N, K;           // N = output columns
+};
+
+// Grouped split-K GEMM used for the weight gradients:
+//   P[grp][split][R, Cc] (fp32) = sum over this split's 64-column slabs of  A[R, k] * B[Cc, k]^T
+// Group grp contracts over columns [k_begin(grp), k_begin(grp) + k_len(grp)) of the two row-major
+// operands; the ranges come from counts[] on the device:
+//   group 0 = [0, pad64(counts[0])),  group 1 = [pad64(counts[0]), + pad64(M - counts[0])).
+struct SplitKArgs {
+  const uint16_t* A; int64_t lda;  // [R, Kpad]
+  const uint16_t* B; int64_t ldb;  // [Cc, Kpad]
+  float* P;                        // [2][splits][R][Cc]
+  const int32_t* counts;
+  int M;                           // routed rows in total (both groups)
+  int R, Cc, splits;
+};
+
+}  // namespace ffnk

@@ -1,0 +1,77 @@
+// Host-side launch interface between the C ABI (capi.hip) and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "gemm_args.hpp"
+
+namespace ffnk {
+
+// ---- route.hip ----
+hipError_t launch_route(const uint8_t* mask, int M, int32_t* perm, int32_t* counts, hipStream_t stream);
+
+// ---- gemm_*.hip: LDS-tiled MFMA kernels ----
+enum TileId : int {
+  TILE_256x256_W8 = 0,  // 256x256 macro tile, 8 waves (2x4), wave tile 128x64
+  TILE_256x256_W4 = 1,  // 256x256 macro tile, 4 waves (2x2), wave tile 128x128
+  TILE_128x128_W4 = 2,  // 128x128 macro tile, 4 waves (2x2), wave tile 64x64
+  TILE_SMALL_W4 = 3,    // 128x64 (plain) or 64x128 holding 64 gate + 64 up rows (SwiGLU), 4 waves
+  TILE_COUNT = 4
+};
+
+// Geometry of a tile id, as reported through ffnk_tile_config().
+struct TileGeom {
+  int block_m, block_n_out, waves_m, waves_n;
+};
+TileGeom tile_geom(int tile, bool dual);
+
+// y = route-gather(x) @ W_g^T, scattered back to token order (MaskedLinear forward, and dx).
+hipError_t launch_linear_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream);
+// H(routed order) = silu(gather(x) @ W1_g^T) * (gather(x) @ W3_g^T)
+hipError_t launch_up_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream);
+// out(token order) = H(routed order) @ W2_g^T
+hipError_t launch_down_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream);
+// P[grp][split] = A[:, kslice] @ B[:, kslice]^T (fp32 partials; weight gradients)
+hipError_t launch_splitk_gemm(int tile, const SplitKArgs& g, hipStream_t stream);
+
+// ---- prep.hip: layout passes around the GEMMs ----
+// dst[r, c] (row-major, ld_dst) = src[r * sr + c * sc] for r < rows, c < cols.
+hipError_t launch_strided_copy2d(const uint16_t* src, int64_t sr, int64_t sc, uint16_t* dst, int64_t ld_dst,
+                                 int rows, int cols, hipStream_t stream);
+// dst[c, pos(p)] = src[perm[p], c]; routed columns padded per group to a multiple of 64 with
+// zeros: pos(p) = p for visual p, pad64(n_vis) + (p - n_vis) for text p.  dst is [cols, ld_dst].
+hipError_t launch_gather_transpose(const uint16_t* src, int64_t ld_src, const int32_t* perm,
+                                   const int32_t* counts, uint16_t* dst, int64_t ld_dst, int M, int cols,
+                                   hipStream_t stream);
+// out_g[r * sr + c * sc] = bf16(sum_s P[g][s][r][c]) for g in {0, 1}.
+hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint16_t* out0, uint16_t* out1,
+                                int64_t sr, int64_t sc, hipStream_t stream);
+
+// ---- generic.hip: any-stride scalar kernels ----
+struct GenericLinearArgs {
+  const uint16_t* x; int64_t sxm, sxk;
+  const uint16_t* W[2]; int64_t swk, swn;  // [visual, text]
+  const uint8_t* mask;
+  uint16_t* y; int64_t sym, syn;
+  int M, K, N;
+};
+hipError_t launch_generic_linear(const GenericLinearArgs& a, hipStream_t stream);
+struct GenericUpArgs {
+  const uint16_t* x; int64_t sxm;
+  const uint16_t* G[2]; const uint16_t* U[2]; int64_t swk, swn;  // gate = W1/U1, up = W3/U3
+  const uint8_t* mask;
+  uint16_t* H; int64_t ldh;
+  int M, K, N;
+};
+hipError_t launch_generic_up(const GenericUpArgs& a, hipStream_t stream);
+struct GenericBwdArgs {
+  const uint16_t* g; int64_t sgm;
+  const uint16_t* x; int64_t sxm;
+  const uint16_t* W[2]; int64_t swk, swn;
+  const uint8_t* mask;
+  uint16_t* dx; int64_t sdxm;
+  uint16_t* dW[2]; int64_t sdk, sdn;
+  int M, K, N;
+};
+hipError_t launch_generic_bwd(const GenericBwdArgs& a, hipStream_t stream);
+
+}  // namespace ffnk

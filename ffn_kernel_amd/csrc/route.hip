@@ -1,0 +1,119 @@
+// Row partition by modality: mask[M] -> perm[M] (visual rows first, each group in ascending
+// row order) and counts[2].  The reference tests mask rows inside every GEMM tile
+// (ffn_kernel/linear.py:120-149); here the same row -> weight assignment is made once,
+// as an integer permutation, so that GEMM tiles never mix modalities.
+//
+// One launch, no inter-block dependency: every block re-counts the visual rows that
+// precede its chunk (and the total) straight from the mask, which is at most M bytes of
+// L2-resident reads per block, then places its own CHUNK rows.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace ffnk {
+
+constexpr int kRouteThreads = 256;
+constexpr int kRouteRowsPerThread = 16;
+constexpr int kRouteChunk = kRouteThreads * kRouteRowsPerThread;  // 4096 rows per block
+
+// 16-bit mask of the non-zero bytes of a 16-byte vector (bit j = byte j).
+__device__ __forceinline__ uint32_t nonzero_bytes16(uint4 v) {
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  uint32_t bits = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint32_t t = (w[i] | ((w[i] & 0x7f7f7f7fu) + 0x7f7f7f7fu)) & 0x80808080u;  // bit 7 of each non-zero byte
+    uint32_t nib = (((t >> 7) * 0x01020408u) >> 24) & 0xFu;                     // gather to 4 bits
+    bits |= nib << (4 * i);
+  }
+  return bits;
+}
+
+// Bits [lo, hi) of a 16-bit field, lo/hi clamped to [0, 16].
+__device__ __forceinline__ uint32_t range_bits16(int64_t lo, int64_t hi) {
+  int l = lo < 0 ? 0 : (lo > 16 ? 16 : (int)lo);
+  int h = hi < 0 ? 0 : (hi > 16 ? 16 : (int)hi);
+  if (h <= l) return 0;
+  return ((1u << h) - 1u) & ~((1u << l) - 1u);
+}
+
+__global__ __launch_bounds__(kRouteThreads) void route_kernel(const uint8_t* __restrict__ mask, int M,
+                                                               int32_t* __restrict__ perm,
+                                                               int32_t* __restrict__ counts) {
+  __shared__ int s_red[2][kRouteThreads / kWave];
+  __shared__ int s_scan[kRouteThreads];
+  const int t = threadIdx.x;
+  const int64_t lo = (int64_t)blockIdx.x * kRouteChunk;  // first row of this block's chunk
+
+  // Phase 1: total visual rows, and visual rows before `lo`, from aligned 16-byte reads.
+  const int a = (int)(reinterpret_cast<uintptr_t>(mask) & 15);
+  const uint4* base = reinterpret_cast<const uint4*>(mask - a);
+  const int64_t nvec = M > 0 ? ((int64_t)a + M + 15) / 16 : 0;  // M == 0: mask may be NULL
+  int tot = 0, bef = 0;
+  for (int64_t v = t; v < nvec; v += kRouteThreads) {
+    const int64_t f = v * 16 - a;  // row index of byte 0 of this vector
+    const uint32_t bits = nonzero_bytes16(base[v]) & range_bits16(-f, (int64_t)M - f);
+    tot += __popc(bits);
+    bef += __popc(bits & range_bits16(-f, lo - f));
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    tot += __shfl_down(tot, off);
+    bef += __shfl_down(bef, off);
+  }
+  if ((t & (kWave - 1)) == 0) {
+    s_red[0][t / kWave] = tot;
+    s_red[1][t / kWave] = bef;
+  }
+  __syncthreads();
+  tot = 0;
+  bef = 0;
+#pragma unroll
+  for (int w = 0; w < kRouteThreads / kWave; ++w) {
+    tot += s_red[0][w];
+    bef += s_red[1][w];
+  }
+  if (blockIdx.x == 0 && t == 0) {
+    counts[0] = tot;
+    counts[1] = M - tot;
+  }
+
+  // Phase 2: this thread owns rows [r0, r0 + 16) of the chunk.
+  const int64_t r0 = lo + (int64_t)t * kRouteRowsPerThread;
+  uint32_t bits = 0;
+#pragma unroll
+  for (int j = 0; j < kRouteRowsPerThread; ++j) {
+    if (r0 + j < M && mask[r0 + j] != 0) bits |= 1u << j;
+  }
+  const int c = __popc(bits);
+  s_scan[t] = c;
+  __syncthreads();
+  // Inclusive Hillis-Steele scan over 256 per-thread counts.
+  for (int off = 1; off < kRouteThreads; off <<= 1) {
+    int add = (t >= off) ? s_scan[t - off] : 0;
+    __syncthreads();
+    s_scan[t] += add;
+    __syncthreads();
+  }
+  int vb = bef + s_scan[t] - c;  // visual rows before r0
+#pragma unroll
+  for (int j = 0; j < kRouteRowsPerThread; ++j) {
+    const int64_t r = r0 + j;
+    if (r < M) {
+      if (bits & (1u << j)) {
+        perm[vb] = (int32_t)r;
+        ++vb;
+      } else {
+        perm[tot + (int)(r - vb)] = (int32_t)r;
+      }
+    }
+  }
+}
+
+hipError_t launch_route(const uint8_t* mask, int M, int32_t* perm, int32_t* counts, hipStream_t stream) {
+  // M == 0 still runs one block so that counts[] is written.
+  const int blocks = M > 0 ? cdiv(M, kRouteChunk) : 1;
+  hipLaunchKernelGGL(route_kernel, dim3(blocks), dim3(kRouteThreads), 0, stream, mask, M, perm, counts);
+  return hipGetLastError();
+}
+
+}  // namespace ffnk

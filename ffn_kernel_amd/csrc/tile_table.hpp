@@ -1,0 +1,49 @@
+// gfx950 tile table: which kernel family and macro tile each (op, M, K, N) uses.
+//
+// The reference looks its tile up with find_spec(table, M // 1024) in A100-tuned JSON files
+// holding one entry each (ffn_kernel/utils.py:3-5, ffn_kernel/bf16_linear_fwd.json,
+// bf16_ffn_fwd.json, bf16_linear_bwd.json).  On MI355X the choice is driven by how many
+// workgroups a shape yields against 256 CUs, so the table is keyed on the real extents.
+#pragma once
+#include "launch.hpp"
+#include "common.hpp"
+
+namespace ffnk {
+
+constexpr int kCus = 256;
+
+// Smallest M for which the LDS-tiled path is used by the FFN forward; below it the
+// weight-streaming kernels win because the op is bound by reading the weights once.
+constexpr int kStreamMaxM = 64;
+
+struct TileChoice {
+  int tile;    // TileId
+  int splits;  // split-K factor (weight-gradient GEMM only)
+};
+
+// Routed GEMM over M rows and n_out output columns.
+inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual) {
+  auto tiles = [&](int tile) {
+    const TileGeom t = tile_geom(tile, dual);
+    return cdiv64(M, t.block_m) * cdiv64(n_out, t.block_n_out);
+  };
+  if (tiles(TILE_256x256_W8) >= 2 * kCus) return TILE_256x256_W8;  // at least two full waves of 256x256 tiles
+  if (tiles(TILE_128x128_W4) >= kCus) return TILE_128x128_W4;
+  return TILE_SMALL_W4;
+}
+
+// Weight-gradient GEMM: two [R, Cc] outputs, contraction over about M / 2 rows each.
+inline TileChoice pick_splitk_tile(int64_t M, int64_t R, int64_t Cc) {
+  TileChoice c;
+  c.tile = TILE_128x128_W4;
+  const int64_t tiles = 2 * cdiv64(R, 128) * cdiv64(Cc, 128);
+  int64_t s = cdiv64(2 * kCus, tiles);            // aim at two workgroups per CU
+  const int64_t slabs = cdiv64(cdiv64(M, 2), 64);  // 64-row slabs per group at an even split
+  if (s > slabs) s = slabs;
+  if (s > 16) s = 16;
+  if (s < 1) s = 1;
+  c.splits = (int)s;
+  return c;
+}
+
+}  // namespace ffnk

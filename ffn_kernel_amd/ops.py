@@ -1,0 +1,227 @@
+"""MaskedLinear / MaskedFFN — the torch.autograd.Function surface of the reference
+(ffn_kernel/ops.py:9-38) on top of libffnk's HIP kernels.
+
+Same class names, same positional signatures:
+    MaskedLinear.apply(a, b1, b2, mask) -> c            b1 = W_v^T, b2 = W_t^T, views [K, N]
+    MaskedFFN.apply(a, w1, w2, w3, u1, u2, u3, mask)    w1, w3, u1, u3 = [d, h]; w2, u2 = [h, d]
+`mask` is a bool [M] tensor: True rows use b1 / w*, False rows use b2 / u*.
+"""
+from __future__ import annotations
+
+import torch
+from torch.autograd import Function
+from torch.autograd.function import once_differentiable
+
+from . import _lib
+
+
+def _require_cuda_bf16(name: str, t: torch.Tensor, ndim: int) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+    if t.dim() != ndim:
+        raise ValueError(f"{name} must be {ndim}-D, got shape {tuple(t.shape)}")
+    if t.dtype != torch.bfloat16:
+        raise ValueError(f"{name} must be torch.bfloat16, got {t.dtype}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on a GPU (got {t.device}); libffnk has no CPU path")
+
+
+def _require_mask(mask: torch.Tensor, M: int, dev: torch.device) -> torch.Tensor:
+    if not isinstance(mask, torch.Tensor) or mask.dtype != torch.bool:
+        raise ValueError(f"mask must be a torch.bool tensor, got {getattr(mask, 'dtype', type(mask))}")
+    if mask.dim() != 1 or mask.shape[0] != M:
+        raise ValueError(f"mask must have shape [{M}], got {tuple(mask.shape)}")
+    if mask.device != dev:
+        raise ValueError(f"mask is on {mask.device}, inputs on {dev}")
+    return mask if mask.stride(0) == 1 or M <= 1 else mask.contiguous()
+
+
+def _rows_contiguous(t: torch.Tensor) -> torch.Tensor:
+    """[M, K] with unit column stride (what the reference's a.contiguous() guarantees,
+    linear.py:430) — row-strided views are passed through without a copy."""
+    if t.shape[1] <= 1 or t.stride(1) == 1:
+        if t.shape[0] <= 1 or t.stride(0) >= t.shape[1]:
+            return t
+    return t.contiguous()
+
+
+def _k_major(w: torch.Tensor) -> torch.Tensor:
+    """Logical [K, N] weight whose memory is [N, K] row-major (stride(0) == 1), the layout of
+    nn.Linear.weight.T that the MFMA path reads directly.  Any other layout is re-laid once."""
+    K, N = w.shape
+    if (K <= 1 or w.stride(0) == 1) and (N <= 1 or w.stride(1) >= K):
+        return w
+    return w.t().contiguous().t()
+
+
+def _same_device(dev, **tensors) -> None:
+    for name, t in tensors.items():
+        if t.device != dev:
+            raise ValueError(f"{name} is on {t.device}, expected {dev}")
+
+
+def _stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _workspace(nbytes: int, dev: torch.device) -> torch.Tensor:
+    # torch's caching allocator hands out 512-byte aligned blocks.
+    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+
+
+def _wstrides(w: torch.Tensor):
+    """(stride_k, stride_n) of a logical [K, N] weight with size-1 dimensions normalised."""
+    K, N = w.shape
+    sk = w.stride(0) if K > 1 else 1
+    sn = w.stride(1) if N > 1 else max(K, 1)
+    if sk == 1 and sn < K:  # both extents ambiguous only when a dimension is 1
+        sn = K
+    return sk, sn
+
+
+def masked_linear_forward(a: torch.Tensor, b1: torch.Tensor, b2: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+    """c[m] = a[m] @ (b1 if mask[m] else b2).  Replaces _bf16_linear_forward (linear.py:418-452)."""
+    _require_cuda_bf16("a", a, 2)
+    _require_cuda_bf16("b1", b1, 2)
+    _require_cuda_bf16("b2", b2, 2)
+    M, K = a.shape
+    if b1.shape[0] != K or b2.shape != b1.shape:
+        raise ValueError(f"weight shapes {tuple(b1.shape)}, {tuple(b2.shape)} do not match a {tuple(a.shape)}")
+    N = b1.shape[1]
+    dev = a.device
+    _same_device(dev, b1=b1, b2=b2)
+    mask = _require_mask(mask, M, dev)
+    a = _rows_contiguous(a)
+    b1, b2 = _k_major(b1), _k_major(b2)
+    if _wstrides(b1) != _wstrides(b2):
+        b2 = b2.t().contiguous().t()
+        b1 = b1.t().contiguous().t()
+    sk, sn = _wstrides(b1)
+    c = torch.empty((M, N), device=dev, dtype=torch.bfloat16)
+    if M == 0 or N == 0:
+        return c
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        ws_bytes = _lib.workspace_bytes(_lib.OP_LINEAR_FWD, M, K, N)
+        ws = _workspace(ws_bytes, dev)
+        rc = lib.ffnk_masked_linear_fwd(a.data_ptr(), a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(),
+                                        b2.data_ptr(), sk, sn, mask.data_ptr(), c.data_ptr(), N, M, K, N,
+                                        ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+    _lib.check(rc, "ffnk_masked_linear_fwd")
+    return c
+
+
+def masked_linear_backward(grad: torch.Tensor, a: torch.Tensor, b1: torch.Tensor, b2: torch.Tensor,
+                           mask: torch.Tensor):
+    """(da, db1, db2) of MaskedLinear.  Replaces _bf16_linear_backward (linear.py:455-496);
+    db1/db2 keep b1's strides as the reference's empty_like(b1) does (linear.py:475)."""
+    _require_cuda_bf16("grad", grad, 2)
+    _require_cuda_bf16("a", a, 2)
+    M, K = a.shape
+    N = b1.shape[1]
+    if grad.shape != (M, N):
+        raise ValueError(f"grad shape {tuple(grad.shape)} != {(M, N)}")
+    dev = a.device
+    mask = _require_mask(mask, M, dev)
+    grad = _rows_contiguous(grad)
+    a = _rows_contiguous(a)
+    if _wstrides(b1) != _wstrides(b2):
+        b2 = b2.t().contiguous().t()
+        b1 = b1.t().contiguous().t()
+    sk, sn = _wstrides(b1)
+    da = torch.empty((M, K), device=dev, dtype=torch.bfloat16)
+    db1, db2 = torch.empty_like(b1), torch.empty_like(b2)
+    if db1.stride() != db2.stride():
+        db2 = torch.empty_strided(db1.shape, db1.stride(), device=dev, dtype=torch.bfloat16)
+    dsk, dsn = _wstrides(db1)
+    if K == 0:
+        return da, db1, db2
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        ws_bytes = _lib.workspace_bytes(_lib.OP_LINEAR_BWD, M, K, N)
+        ws = _workspace(ws_bytes, dev)
+        rc = lib.ffnk_masked_linear_bwd(grad.data_ptr(), grad.stride(0) if M > 1 else max(N, 1), a.data_ptr(),
+                                        a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(), b2.data_ptr(), sk, sn,
+                                        mask.data_ptr(), da.data_ptr(), K, db1.data_ptr(), db2.data_ptr(), dsk,
+                                        dsn, M, K, N, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+    _lib.check(rc, "ffnk_masked_linear_bwd")
+    return da, db1, db2
+
+
+def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask) -> torch.Tensor:
+    """SwiGLU FFN routed by mask.  Replaces _bf16_ffn_forward + _bf16_linear_forward
+    (ops.py:30-32, ffn.py:527-560)."""
+    _require_cuda_bf16("a", a, 2)
+    for name, w in (("w1", w1), ("w2", w2), ("w3", w3), ("u1", u1), ("u2", u2), ("u3", u3)):
+        _require_cuda_bf16(name, w, 2)
+    M, d = a.shape
+    h = w1.shape[1]
+    for name, w in (("w1", w1), ("w3", w3), ("u1", u1), ("u3", u3)):
+        if w.shape != (d, h):
+            raise ValueError(f"{name} shape {tuple(w.shape)} != {(d, h)}")
+    for name, w in (("w2", w2), ("u2", u2)):
+        if w.shape[0] != h or w.shape != w2.shape:
+            raise ValueError(f"{name} shape {tuple(w.shape)} does not match [h={h}, out]")
+    d_out = w2.shape[1]
+    if d_out != d:
+        # The C entry point fuses both stages for the square case only; chain the two ops otherwise.
+        raise ValueError(f"MaskedFFN needs w2/u2 of shape [{h}, {d}], got {tuple(w2.shape)}")
+    dev = a.device
+    _same_device(dev, w1=w1, w2=w2, w3=w3, u1=u1, u2=u2, u3=u3)
+    mask = _require_mask(mask, M, dev)
+    a = _rows_contiguous(a)
+    ups = [_k_major(w) for w in (w1, w3, u1, u3)]
+    if len({_wstrides(w) for w in ups}) != 1:
+        ups = [w.t().contiguous().t() for w in ups]
+    downs = [_k_major(w) for w in (w2, u2)]
+    if len({_wstrides(w) for w in downs}) != 1:
+        downs = [w.t().contiguous().t() for w in downs]
+    usk, usn = _wstrides(ups[0])
+    dsk, dsn = _wstrides(downs[0])
+    out = torch.empty((M, d), device=dev, dtype=torch.bfloat16)
+    if M == 0 or d == 0:
+        return out
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_FWD, M, d, h)
+        ws = _workspace(ws_bytes, dev)
+        rc = lib.ffnk_masked_ffn_fwd(a.data_ptr(), a.stride(0) if M > 1 else max(d, 1), ups[0].data_ptr(),
+                                     ups[1].data_ptr(), ups[2].data_ptr(), ups[3].data_ptr(), usk, usn,
+                                     downs[0].data_ptr(), downs[1].data_ptr(), dsk, dsn, mask.data_ptr(),
+                                     out.data_ptr(), d, M, d, h, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+    _lib.check(rc, "ffnk_masked_ffn_fwd")
+    return out
+
+
+class MaskedLinear(Function):
+    """c = a @ (b1 where mask else b2), forward and backward (reference: ops.py:9-24)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, a, b1, b2, mask):
+        ctx.save_for_backward(a, mask)
+        ctx.b1, ctx.b2 = b1, b2
+        return masked_linear_forward(a, b1, b2, mask)
+
+    @staticmethod
+    @once_differentiable
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad):
+        a, mask = ctx.saved_tensors
+        da, db1, db2 = masked_linear_backward(grad, a, ctx.b1, ctx.b2, mask)
+        return da, db1, db2, None
+
+
+class MaskedFFN(Function):
+    """Routed SwiGLU FFN, forward only like the reference (ops.py:27-38)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, a, w1, w2, w3, u1, u2, u3, mask):
+        return masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask)
+
+    @staticmethod
+    @once_differentiable
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad):
+        raise NotImplementedError

@@ -1,0 +1,161 @@
+/*
+ * ffnk.h — C ABI of libffnk.so: mask-routed bf16 linear / SwiGLU-FFN kernels for
+ * AMD MI355X (gfx950).
+ *
+ * This is the boundary the reference crosses when its Python launchers start a Triton
+ * kernel (ffn_kernel/linear.py:418-452, 455-496; ffn_kernel/ffn.py:527-560).  Every
+ * pointer below is a DEVICE pointer unless its comment says otherwise.  Every entry
+ * point only enqueues work on `stream` (a hipStream_t passed as void*, NULL = the
+ * null stream): no host synchronisation, no allocation, no free.  Scratch memory is
+ * supplied by the caller through (`ws`, `ws_bytes`); its required size comes from
+ * ffnk_workspace_bytes().
+ *
+ * Return value of every int-returning function: 0 on success; a negative FFNK_E_*
+ * code for a rejected argument; a positive value is a hipError_t from the runtime.
+ * ffnk_last_error() returns a thread-local text for the last non-zero return.
+ *
+ * Tensors are bf16 stored as uint16_t.  `mask` is one byte per token row
+ * (torch.bool storage): non-zero = visual row, zero = text row.
+ */
+#ifndef FFNK_H
+#define FFNK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FFNK_VERSION 100
+
+#if defined(__GNUC__)
+#define FFNK_API __attribute__((visibility("default")))
+#else
+#define FFNK_API
+#endif
+
+enum {
+  FFNK_OK = 0,
+  FFNK_E_NULL = -1,       /* a required pointer is NULL                         */
+  FFNK_E_SHAPE = -2,      /* negative / overflowing / unsupported extent        */
+  FFNK_E_STRIDE = -3,     /* stride combination no kernel here can address      */
+  FFNK_E_ALIGN = -4,      /* pointer not 2-byte aligned                         */
+  FFNK_E_WORKSPACE = -5,  /* ws_bytes smaller than ffnk_workspace_bytes()       */
+  FFNK_E_OP = -6          /* unknown op id                                      */
+};
+
+/* op ids for ffnk_workspace_bytes / ffnk_tile_config */
+enum {
+  FFNK_OP_LINEAR_FWD = 0, /* MaskedLinear forward                (K = in, N = out)  */
+  FFNK_OP_FFN_FWD = 1,    /* MaskedFFN forward                   (K = d,  N = h)    */
+  FFNK_OP_LINEAR_BWD = 2, /* MaskedLinear backward               (K = in, N = out)  */
+  FFNK_OP_FFN_UP = 3,     /* tile_config only: up-projection + SwiGLU stage         */
+  FFNK_OP_FFN_DOWN = 4,   /* tile_config only: down-projection stage                */
+  FFNK_OP_BWD_DX = 5,     /* tile_config only: dx GEMM of the backward              */
+  FFNK_OP_BWD_DW = 6      /* tile_config only: dW GEMM of the backward              */
+};
+
+/* kernel families reported by ffnk_tile_config */
+enum {
+  FFNK_PATH_MFMA_TILED = 0,   /* LDS-staged MFMA macro-tile GEMM (large M)          */
+  FFNK_PATH_STREAM = 1,       /* weight-streaming MFMA kernels (decode, small M)    */
+  FFNK_PATH_GENERIC = 2       /* any-stride scalar kernel (unaligned / odd strides) */
+};
+
+/* One entry of the gfx950 tile table (replaces the reference's find_spec() lookup in
+ * its A100-tuned JSON tables: ffn_kernel/utils.py:3-5, ffn_kernel/bf16_*_fwd.json). */
+typedef struct ffnk_tile_config_t {
+  int32_t path;        /* FFNK_PATH_*                                              */
+  int32_t block_m;     /* token rows per workgroup tile                            */
+  int32_t block_n;     /* output columns per workgroup tile                        */
+  int32_t block_k;     /* contraction elements per LDS stage / per streamed chunk  */
+  int32_t waves_m;     /* wavefront grid inside the workgroup                      */
+  int32_t waves_n;
+  int32_t lds_stages;  /* LDS buffers in flight                                    */
+  int32_t group_m;     /* M-tiles per L2 super-group in the tile order             */
+  int32_t split_k;     /* contraction splits reduced by a second kernel (1 = none) */
+  int32_t direct_lds;  /* 1 = global->LDS loads bypass registers                   */
+} ffnk_tile_config_t;
+
+FFNK_API int ffnk_version(void);
+
+/* Text for the calling thread's last non-zero return ("" if none). Never NULL. */
+FFNK_API const char* ffnk_last_error(void);
+
+/*
+ * Row partition.  Writes perm[0..M) = indices of visual rows in ascending order followed
+ * by indices of text rows in ascending order (a stable partition of 0..M-1 by mask), and
+ * counts[0] = number of visual rows, counts[1] = number of text rows.
+ * No counterpart kernel in the reference (it routes per tile, ffn_kernel/linear.py:120-149);
+ * it yields the same row -> weight assignment as the mask test there.
+ */
+FFNK_API int ffnk_route(const uint8_t* mask, int64_t M, int32_t* perm, int32_t* counts, void* stream);
+
+/* Bytes of scratch the op needs for these extents (0 is a valid answer).
+ * Returns (size_t)-1 for an unknown op or invalid extents. */
+FFNK_API size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N);
+
+/* Which tile-table entry the library uses for these extents. */
+FFNK_API int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t* out);
+
+/*
+ * MaskedLinear forward — replaces _bf16_linear_forward (ffn_kernel/linear.py:418-452):
+ *   y[m, :] = x[m, :] @ (mask[m] ? Wv : Wt)      for m in [0, M)
+ * x: [M, K], element strides (x_stride_m, 1).  Wv, Wt: logical [K, N] with element strides
+ * (w_stride_k, w_stride_n) as in the reference call (b1.stride(0), b1.stride(1),
+ * linear.py:442-443); nn.Linear.weight.T gives (1, K).  y: [M, N] strides (y_stride_m, 1).
+ * Accumulation is fp32; the result is rounded to bf16 once.
+ */
+FFNK_API int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m,
+                           const uint16_t* Wv, const uint16_t* Wt,
+                           int64_t w_stride_k, int64_t w_stride_n,
+                           const uint8_t* mask,
+                           uint16_t* y, int64_t y_stride_m,
+                           int64_t M, int64_t K, int64_t N,
+                           void* ws, size_t ws_bytes, void* stream);
+
+/*
+ * MaskedFFN forward — replaces _bf16_ffn_forward followed by _bf16_linear_forward
+ * (ffn_kernel/ops.py:30-32, ffn_kernel/ffn.py:527-560):
+ *   visual row:  out = (silu(x W1) * (x W3)) W2        text row: same with U1, U3, U2
+ * W1, W3, U1, U3: logical [d, h] with strides (up_stride_k, up_stride_n) shared by all four
+ * (ffn.py:551); W2, U2: logical [h, d] with strides (down_stride_k, down_stride_n).
+ * The [M, h] intermediate is rounded to bf16 once (as the reference stores it, ffn.py:113).
+ * Picks the macro-tile path or the weight-streaming path from M.
+ */
+FFNK_API int ffnk_masked_ffn_fwd(const uint16_t* x, int64_t x_stride_m,
+                        const uint16_t* W1, const uint16_t* W3,
+                        const uint16_t* U1, const uint16_t* U3,
+                        int64_t up_stride_k, int64_t up_stride_n,
+                        const uint16_t* W2, const uint16_t* U2,
+                        int64_t down_stride_k, int64_t down_stride_n,
+                        const uint8_t* mask,
+                        uint16_t* out, int64_t out_stride_m,
+                        int64_t M, int64_t d, int64_t h,
+                        void* ws, size_t ws_bytes, void* stream);
+
+/*
+ * MaskedLinear backward — replaces _bf16_linear_backward (ffn_kernel/linear.py:455-496):
+ *   dx[m, :]  = g[m, :] @ (mask[m] ? Wv : Wt)^T
+ *   dWv       = x[visual rows]^T @ g[visual rows]       (exact zeros if there are none)
+ *   dWt       = x[text rows]^T   @ g[text rows]
+ * g: [M, N] strides (g_stride_m, 1); x: [M, K]; Wv/Wt as in the forward; dx: [M, K];
+ * dWv, dWt: logical [K, N] with strides (dw_stride_k, dw_stride_n) (the reference
+ * allocates them with empty_like(b1), linear.py:475).  Deterministic: no atomics.
+ */
+FFNK_API int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m,
+                           const uint16_t* x, int64_t x_stride_m,
+                           const uint16_t* Wv, const uint16_t* Wt,
+                           int64_t w_stride_k, int64_t w_stride_n,
+                           const uint8_t* mask,
+                           uint16_t* dx, int64_t dx_stride_m,
+                           uint16_t* dWv, uint16_t* dWt,
+                           int64_t dw_stride_k, int64_t dw_stride_n,
+                           int64_t M, int64_t K, int64_t N,
+                           void* ws, size_t ws_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FFNK_H */

@@ -1,0 +1,292 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle.
+
+Tolerance (floating point): max-abs <= 2e-2 (or <= 1 bf16 ulp of the reference where bf16 cannot
+resolve 2e-2) and rel-L2 <= 5e-3 against a double-precision reference.  Routing is bit-exact.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from ffn_kernel_amd import MaskedFFN, MaskedLinear, _lib
+from ffn_kernel_amd import workloads as wl
+from oracle import cref
+from oracle import modules as om
+from helpers import assert_close, note
+
+pytestmark = pytest.mark.gpu
+
+
+# ------------------------------------------------------------------ routing (integer, bit-exact)
+@pytest.mark.parametrize("M", [0, 1, 2, 15, 16, 17, 63, 64, 65, 255, 4095, 4096, 4097, 10000, 32768, 100003])
+@pytest.mark.parametrize("p", [0.0, 0.5, 1.0])
+def test_route_bit_exact(dev, M, p):
+    note(f"route M={M} p={p}")
+    gen = torch.Generator().manual_seed(M * 7 + int(p * 10))
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    perm_ref, counts_ref = om.stable_partition(mask.numpy())
+    mask_d = mask.to(dev)
+    perm = torch.full((max(M, 1),), -1, dtype=torch.int32, device=dev)
+    counts = torch.full((2,), -1, dtype=torch.int32, device=dev)
+    rc = _lib.load().ffnk_route(mask_d.data_ptr() if M else None, M, perm.data_ptr(), counts.data_ptr(),
+                                torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "ffnk_route")
+    torch.cuda.synchronize()
+    assert counts.cpu().numpy().tolist() == counts_ref.tolist()
+    assert np.array_equal(perm.cpu().numpy()[:M], perm_ref)
+
+
+def test_route_unaligned_mask_view(dev):
+    note("route on a mask view that starts at an odd byte")
+    gen = torch.Generator().manual_seed(5)
+    big = (torch.rand(9000, generator=gen) < 0.4).to(dev)
+    for off in (1, 3, 7, 13):
+        mask = big[off:off + 8191]
+        perm_ref, counts_ref = om.stable_partition(mask.cpu().numpy())
+        perm = torch.empty(8191, dtype=torch.int32, device=dev)
+        counts = torch.empty(2, dtype=torch.int32, device=dev)
+        _lib.check(_lib.load().ffnk_route(mask.data_ptr(), 8191, perm.data_ptr(), counts.data_ptr(),
+                                          torch.cuda.current_stream().cuda_stream), "ffnk_route")
+        assert counts.cpu().numpy().tolist() == counts_ref.tolist()
+        assert np.array_equal(perm.cpu().numpy(), perm_ref)
+
+
+# ------------------------------------------------------------------ MaskedLinear forward
+def _run_linear(w, dev):
+    d = w.to(dev)
+    y = MaskedLinear.apply(d.x, d.Wv.T, d.Wt.T, d.mask)
+    torch.cuda.synchronize()
+    return y
+
+
+LINEAR_SHAPES = [
+    # (M, K, N, p_visual)            what it exercises
+    (37, 48, 40, 0.5),               # tiny, ragged everything, K tail (register-staged loads)
+    (1, 64, 64, 1.0),                # single visual row
+    (1, 64, 64, 0.0),                # single text row
+    (129, 64, 200, 0.3),             # direct loads, ragged N
+    (300, 128, 136, 0.7),            # partial tiles in both groups
+    (513, 1024, 1024, 0.5),          # Bernoulli mask
+    (2048, 1024, 1024, -1),          # cfg1 (span mask)
+    (4096, 512, 2048, 0.5),          # 256x256 tile family
+    (1000, 72, 264, 0.5),            # K % 64 != 0, K % 8 == 0
+]
+
+
+@pytest.mark.parametrize("M,K,N,p", LINEAR_SHAPES)
+def test_linear_fwd_vs_oracle(dev, M, K, N, p):
+    note(f"linear fwd M={M} K={K} N={N} p={p}")
+    if p < 0:
+        w = wl.cfg1_linear_fwd()
+    else:
+        gen = torch.Generator().manual_seed(M + K + N)
+        mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+        w = wl.make_linear("t", M, K, N, mask, seed=M)
+    y = _run_linear(w, dev)
+    assert y.dtype == torch.bfloat16 and y.shape == (M, N)
+    ref = cref.linear_fwd(w.x, w.Wv, w.Wt, w.mask)
+    assert_close(y, ref, f"linear fwd {M}x{K}x{N}")
+    # and against the reference's own (blend-form, bf16) PyTorch module maths
+    blend = om.linear_blend(w.x, w.Wv, w.Wt, w.mask)
+    assert_close(y, blend.double(), "vs blend-form bf16 module")
+
+
+def test_linear_row_selection_is_exact(dev):
+    """W_v = I, W_t = 2 I: every output row equals x or 2 x bit for bit."""
+    note("linear identity weights")
+    M, K = 777, 256
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    mask = torch.rand(M, generator=gen) < 0.5
+    eye = torch.eye(K).to(torch.bfloat16)
+    y = MaskedLinear.apply(x.to(dev), eye.to(dev).T, (2 * eye).to(dev).T, mask.to(dev)).cpu()
+    expect = torch.where(mask[:, None], x, 2 * x)
+    assert torch.equal(y, expect)
+
+
+def test_linear_unused_branch_never_touched(dev):
+    """Poisoning the text weight with NaN must leave visual rows finite (the blend form would not)."""
+    note("linear NaN poison")
+    M, K, N = 300, 128, 128
+    gen = torch.Generator().manual_seed(4)
+    mask = torch.rand(M, generator=gen) < 0.5
+    w = wl.make_linear("t", M, K, N, mask, seed=9)
+    Wt = torch.full_like(w.Wt, float("nan"))
+    y = MaskedLinear.apply(w.x.to(dev), w.Wv.to(dev).T, Wt.to(dev).T, mask.to(dev)).cpu()
+    assert torch.isfinite(y[mask]).all()
+    assert torch.isnan(y[~mask]).all()
+    ref = cref.linear_fwd(w.x, w.Wv, w.Wt, torch.ones(M, dtype=torch.bool))
+    assert_close(y[mask], ref[mask], "visual rows")
+
+
+def test_linear_row_permutation_equivariance(dev):
+    """Permuting rows of (x, mask) permutes the output rows bit for bit."""
+    note("linear permutation equivariance")
+    M, K, N = 1000, 256, 320
+    gen = torch.Generator().manual_seed(8)
+    mask = torch.rand(M, generator=gen) < 0.4
+    w = wl.make_linear("t", M, K, N, mask, seed=2).to(dev)
+    y = MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, w.mask)
+    pi = torch.randperm(M, generator=gen).to(dev)
+    y2 = MaskedLinear.apply(w.x[pi].contiguous(), w.Wv.T, w.Wt.T, w.mask[pi].contiguous())
+    assert torch.equal(y[pi], y2)
+
+
+def test_linear_generic_path_odd_shapes(dev):
+    """K not a multiple of 8 and a [K, N]-contiguous weight go through other code paths."""
+    note("linear generic path")
+    for (M, K, N) in [(50, 30, 17), (9, 1, 5), (64, 100, 3)]:
+        gen = torch.Generator().manual_seed(M)
+        mask = torch.rand(M, generator=gen) < 0.5
+        w = wl.make_linear("t", M, K, N, mask, seed=M)
+        y = _run_linear(w, dev)
+        assert_close(y, cref.linear_fwd(w.x, w.Wv, w.Wt, w.mask), f"generic {M}x{K}x{N}")
+    # weight given as a contiguous [K, N] tensor (stride (N, 1)): re-laid once by the op
+    M, K, N = 256, 128, 192
+    mask = torch.rand(M, generator=torch.Generator().manual_seed(1)) < 0.5
+    w = wl.make_linear("t", M, K, N, mask, seed=5)
+    d = w.to(dev)
+    y = MaskedLinear.apply(d.x, d.Wv.T.contiguous(), d.Wt.T.contiguous(), d.mask)
+    assert_close(y, cref.linear_fwd(w.x, w.Wv, w.Wt, w.mask), "[K,N]-contiguous weights")
+
+
+def test_linear_strided_x_and_empty(dev):
+    note("linear strided x / empty")
+    M, K, N = 200, 64, 128
+    mask = torch.rand(M, generator=torch.Generator().manual_seed(1)) < 0.5
+    w = wl.make_linear("t", M, K, N, mask, seed=6)
+    wide = torch.zeros(M, 2 * K, dtype=torch.bfloat16, device=dev)
+    wide[:, :K] = w.x.to(dev)
+    y = MaskedLinear.apply(wide[:, :K], w.Wv.to(dev).T, w.Wt.to(dev).T, mask.to(dev))
+    assert_close(y, cref.linear_fwd(w.x, w.Wv, w.Wt, w.mask), "row-strided x")
+    y0 = MaskedLinear.apply(torch.empty(0, K, dtype=torch.bfloat16, device=dev), w.Wv.to(dev).T, w.Wt.to(dev).T,
+                            torch.empty(0, dtype=torch.bool, device=dev))
+    assert y0.shape == (0, N)
+
+
+# ------------------------------------------------------------------ MaskedFFN forward
+FFN_SHAPES = [
+    (19, 32, 48, 0.5),        # K tails in both stages
+    (1, 64, 128, 1.0),
+    (1, 64, 128, 0.0),
+    (8, 256, 512, 0.5),
+    (64, 512, 1024, 0.5),
+    (333, 128, 320, 0.3),
+    (2048, 1024, 2048, 0.5),
+    (50, 36, 20, 0.5),        # generic path (d, h not multiples of 8)
+]
+
+
+@pytest.mark.parametrize("M,d,h,p", FFN_SHAPES)
+def test_ffn_fwd_vs_oracle(dev, M, d, h, p):
+    note(f"ffn fwd M={M} d={d} h={h} p={p}")
+    gen = torch.Generator().manual_seed(M + d + h)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_ffn("t", M, d, h, mask, seed=M, w_std=0.05)
+    out = MaskedFFN.apply(*w.to(dev).op_args())
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16 and out.shape == (M, d)
+    assert_close(out, cref.ffn_fwd(w.x, w.W, w.mask), f"ffn {M}x{d}x{h}")
+    assert_close(out, om.ffn_blend(w.x, w.W, w.mask).double(), "vs blend-form bf16 module")
+
+
+def test_ffn_cfg2(dev):
+    note("ffn cfg2")
+    w = wl.cfg2_ffn_fwd()
+    out = MaskedFFN.apply(*w.to(dev).op_args())
+    # double-precision torch reference on the select form (the C loops would take minutes here)
+    ref = om.ffn_select(w.x, w.W, w.mask, torch.float64)
+    rep = assert_close(out, ref, "cfg2")
+    print("cfg2 error:", rep)
+
+
+def test_ffn_closed_forms(dev):
+    """W3 = 0 or W1 = 0 gives exact zeros on visual rows; text rows unaffected."""
+    note("ffn closed forms")
+    M, d, h = 130, 64, 128
+    mask = torch.rand(M, generator=torch.Generator().manual_seed(2)) < 0.5
+    w = wl.make_ffn("t", M, d, h, mask, seed=3, w_std=0.05)
+    ref = cref.ffn_fwd(w.x, w.W, w.mask)
+    for zero in ("w3", "w1"):
+        W = dict(w.W)
+        W[zero] = torch.zeros_like(W[zero])
+        w2 = wl.FFNWorkload("z", w.x, W, w.mask).to(dev)
+        out = MaskedFFN.apply(*w2.op_args()).cpu()
+        assert (out[mask] == 0).all()
+        assert_close(out[~mask], ref[~mask], "text rows")
+
+
+def test_ffn_backward_raises(dev):
+    note("ffn backward raises")
+    w = wl.make_ffn("t", 8, 64, 64, torch.ones(8, dtype=torch.bool), seed=1).to(dev)
+    x = w.x.clone().requires_grad_(True)
+    args = list(w.op_args())
+    args[0] = x
+    out = MaskedFFN.apply(*args)
+    with pytest.raises(NotImplementedError):
+        out.sum().backward()
+
+
+# ------------------------------------------------------------------ MaskedLinear backward
+BWD_SHAPES = [
+    (37, 48, 40, 0.5),
+    (64, 64, 64, 1.0),        # no text rows: dW_t must be exact zeros
+    (64, 64, 64, 0.0),
+    (300, 128, 136, 0.5),
+    (1000, 256, 320, 0.3),
+    (2048, 1024, 1024, 0.5),
+    (50, 30, 17, 0.5),        # generic path
+]
+
+
+@pytest.mark.parametrize("M,K,N,p", BWD_SHAPES)
+def test_linear_bwd_vs_oracle(dev, M, K, N, p):
+    note(f"linear bwd M={M} K={K} N={N} p={p}")
+    gen = torch.Generator().manual_seed(M + K + N + 1)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_linear("t", M, K, N, mask, seed=M + 1, with_grad=True, w_std=0.05)
+    d = w.to(dev)
+    x = d.x.clone().requires_grad_(True)
+    Wv = d.Wv.clone().requires_grad_(True)
+    Wt = d.Wt.clone().requires_grad_(True)
+    y = MaskedLinear.apply(x, Wv.T, Wt.T, d.mask)
+    y.backward(d.grad)
+    torch.cuda.synchronize()
+    dx, dWv, dWt = cref.linear_bwd(w.grad, w.x, w.Wv, w.Wt, w.mask)
+    assert x.grad.shape == (M, K) and Wv.grad.shape == (N, K) and Wv.grad.is_contiguous()
+    assert_close(x.grad, dx, "dx")
+    assert_close(Wv.grad, dWv, "dWv")
+    assert_close(Wt.grad, dWt, "dWt")
+    if p == 1.0:
+        assert (Wt.grad == 0).all()
+    if p == 0.0:
+        assert (Wv.grad == 0).all()
+
+
+def test_linear_bwd_is_deterministic(dev):
+    note("linear bwd determinism")
+    w = wl.make_linear("t", 1500, 256, 256, torch.rand(1500, generator=torch.Generator().manual_seed(0)) < 0.5,
+                       seed=3, with_grad=True).to(dev)
+    outs = []
+    for _ in range(3):
+        from ffn_kernel_amd import masked_linear_backward
+        outs.append(masked_linear_backward(w.grad, w.x, w.Wv.T, w.Wt.T, w.mask))
+    for o in outs[1:]:
+        for a, b in zip(outs[0], o):
+            assert torch.equal(a, b)
+
+
+def test_linear_bwd_cfg3(dev):
+    note("linear bwd cfg3")
+    w = wl.cfg3_linear_bwd()
+    d = w.to(dev)
+    from ffn_kernel_amd import masked_linear_backward
+    dx, dbv, dbt = masked_linear_backward(d.grad, d.x, d.Wv.T, d.Wt.T, d.mask)
+    rdx, rdWv, rdWt = om.linear_backward_select(w.grad, w.x, w.Wv, w.Wt, w.mask, torch.float64)
+    assert_close(dx, rdx, "dx")
+    assert_close(dbv.T, rdWv, "dWv")
+    assert_close(dbt.T, rdWt, "dWt")
+    # invariant: dW_v + dW_t is the unmasked x^T g
+    tot = (w.grad.double().T @ w.x.double())
+    assert_close((dbv.T.float() + dbt.T.float()), tot, "dWv + dWt == g^T x")
