@@ -27,6 +27,9 @@ _SIGNATURES = {
     "ffnk_masked_ffn_fwd": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                     c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64,
                                     c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "ffnk_masked_ffn_fwd_ev": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                       c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64,
+                                       c_int64, c_int64, c_void_p, c_size_t, c_void_p, c_void_p]),
     "ffnk_masked_linear_bwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64,
                                        c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                        c_int64, c_int64, c_void_p, c_size_t, c_void_p]),

@@ -201,7 +201,20 @@ int ffnk_masked_ffn_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t* W
                         const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
                         const uint8_t* mask, uint16_t* out, int64_t out_stride_m, int64_t M, int64_t d,
                         int64_t h, void* ws, size_t ws_bytes, void* stream_) {
+  return ffnk_masked_ffn_fwd_ev(x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k,
+                                down_stride_n, mask, out, out_stride_m, M, d, h, ws, ws_bytes, stream_, nullptr);
+}
+
+int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, const uint16_t* W3,
+                           const uint16_t* U1, const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n,
+                           const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
+                           const uint8_t* mask, uint16_t* out, int64_t out_stride_m, int64_t M, int64_t d,
+                           int64_t h, void* ws, size_t ws_bytes, void* stream_, void* const* events) {
   hipStream_t stream = (hipStream_t)stream_;
+  auto mark = [&](int i) -> hipError_t {
+    if (events && events[i]) return hipEventRecord((hipEvent_t)events[i], stream);
+    return hipSuccess;
+  };
   if (int e = check_extents(M, d, h)) return e;
   if (M == 0 || d == 0) return FFNK_OK;
   if (!x || !mask || !out) return fail(FFNK_E_NULL, "x, mask or out is NULL");
@@ -230,17 +243,21 @@ int ffnk_masked_ffn_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t* W
     u.G[0] = W1; u.G[1] = U1; u.U[0] = W3; u.U[1] = U3; u.swk = up_stride_k; u.swn = up_stride_n;
     u.mask = mask; u.H = H; u.ldh = ldh;
     u.M = (int)M; u.K = (int)d; u.N = (int)h;
+    FFNK_HIP(mark(0), "event record");
     FFNK_HIP(launch_generic_up(u, stream), "generic up kernel");
+    FFNK_HIP(mark(1), "event record");
     GenericLinearArgs a;
     a.x = H; a.sxm = ldh; a.sxk = 1;
     a.W[0] = W2; a.W[1] = U2; a.swk = down_stride_k; a.swn = down_stride_n;
     a.mask = mask; a.y = out; a.sym = out_stride_m; a.syn = 1;
     a.M = (int)M; a.K = (int)h; a.N = (int)d;
     FFNK_HIP(launch_generic_linear(a, stream), "generic down kernel");
+    FFNK_HIP(mark(2), "event record");
     return FFNK_OK;
   }
 
   FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+  FFNK_HIP(mark(0), "event record");
   GemmArgs up;
   up.A = x; up.lda = x_stride_m;
   up.B0[0] = W1; up.B0[1] = U1; up.B1[0] = W3; up.B1[1] = U3; up.ldb = up_stride_n;
@@ -248,6 +265,7 @@ int ffnk_masked_ffn_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t* W
   up.perm = r.perm; up.counts = r.counts;
   up.M = (int)M; up.N = (int)h; up.K = (int)d;
   FFNK_HIP(launch_up_gemm(pick_routed_tile(M, h, true), d % 64 == 0, up, stream), "up-projection GEMM");
+  FFNK_HIP(mark(1), "event record");
   GemmArgs dn;
   dn.A = H; dn.lda = ldh;
   dn.B0[0] = W2; dn.B0[1] = U2; dn.B1[0] = dn.B1[1] = nullptr; dn.ldb = down_stride_n;
@@ -255,6 +273,7 @@ int ffnk_masked_ffn_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t* W
   dn.perm = r.perm; dn.counts = r.counts;
   dn.M = (int)M; dn.N = (int)d; dn.K = (int)h;
   FFNK_HIP(launch_down_gemm(pick_routed_tile(M, d, false), h % 64 == 0, dn, stream), "down-projection GEMM");
+  FFNK_HIP(mark(2), "event record");
   return FFNK_OK;
 }
 

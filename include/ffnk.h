@@ -136,6 +136,25 @@ FFNK_API int ffnk_masked_ffn_fwd(const uint16_t* x, int64_t x_stride_m,
                         void* ws, size_t ws_bytes, void* stream);
 
 /*
+ * Same as ffnk_masked_ffn_fwd, with stage timing for profilers and benchmarks: `events` is
+ * NULL or a HOST array of three hipEvent_t handles (each may be NULL) that are recorded on
+ * `stream` after the row partition, after the up-projection + SwiGLU stage and after the
+ * down-projection stage.  The caller creates, reads and destroys the events.
+ * No counterpart in the reference (it times whole module calls with an external wall-clock
+ * profiler, test_ffn.py:21-29).
+ */
+FFNK_API int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m,
+                           const uint16_t* W1, const uint16_t* W3,
+                           const uint16_t* U1, const uint16_t* U3,
+                           int64_t up_stride_k, int64_t up_stride_n,
+                           const uint16_t* W2, const uint16_t* U2,
+                           int64_t down_stride_k, int64_t down_stride_n,
+                           const uint8_t* mask,
+                           uint16_t* out, int64_t out_stride_m,
+                           int64_t M, int64_t d, int64_t h,
+                           void* ws, size_t ws_bytes, void* stream, void* const* events);
+
+/*
  * MaskedLinear backward — replaces _bf16_linear_backward (ffn_kernel/linear.py:455-496):
  *   dx[m, :]  = g[m, :] @ (mask[m] ? Wv : Wt)^T
  *   dWv       = x[visual rows]^T @ g[visual rows]       (exact zeros if there are none)

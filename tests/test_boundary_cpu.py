@@ -1,0 +1,95 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol the header
+declares, size/introspection entry points answer, argument validation raises, and the workload
+generators are deterministic."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from ffn_kernel_amd import MaskedFFN, MaskedLinear, _lib
+from ffn_kernel_amd import workloads as wl
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "ffnk.h").read_text()
+    declared = set(re.findall(r"FFNK_API\s+[\w\s\*]+?\b(ffnk_\w+)\s*\(", header))
+    assert declared == set(_lib.EXPORTED_SYMBOLS), declared ^ set(_lib.EXPORTED_SYMBOLS)
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name)
+    assert lib.ffnk_version() == int(re.search(r"#define FFNK_VERSION (\d+)", header).group(1))
+
+
+def test_workspace_bytes():
+    assert _lib.workspace_bytes(_lib.OP_LINEAR_FWD, 0, 8, 8) >= 0
+    a = _lib.workspace_bytes(_lib.OP_LINEAR_FWD, 2048, 1024, 1024)
+    assert a >= 2048 * 4 + 8
+    f = _lib.workspace_bytes(_lib.OP_FFN_FWD, 32768, 4096, 14336)
+    assert f >= 32768 * 14336 * 2  # the bf16 intermediate
+    b = _lib.workspace_bytes(_lib.OP_LINEAR_BWD, 8192, 1024, 1024)
+    assert b >= 2 * 8192 * 1024 * 2  # both transposed operands
+    with pytest.raises(ValueError):
+        _lib.workspace_bytes(99, 1, 1, 1)
+    with pytest.raises(ValueError):
+        _lib.workspace_bytes(_lib.OP_LINEAR_FWD, -1, 1, 1)
+
+
+def test_tile_table_entries():
+    big = _lib.tile_config(_lib.OP_FFN_UP, 32768, 4096, 14336)
+    assert big["path"] == _lib.PATH_MFMA_TILED and big["block_m"] == 256 and big["direct_lds"] == 1
+    assert big["block_k"] == 64 and big["lds_stages"] == 2
+    small = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 1024, 1024)
+    assert small["block_m"] * small["block_n"] < 256 * 256  # small problems get small tiles
+    tail = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 72, 1024)
+    assert tail["direct_lds"] == 0
+    dw = _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)
+    assert dw["split_k"] > 1
+    with pytest.raises(ValueError):
+        _lib.tile_config(77, 1, 1, 1)
+
+
+def test_c_abi_rejects_bad_arguments_without_a_gpu():
+    lib = _lib.load()
+    assert lib.ffnk_route(None, 10, None, None, None) == -1
+    assert b"NULL" in lib.ffnk_last_error()
+    assert lib.ffnk_masked_linear_fwd(None, 8, None, None, 1, 8, None, None, 8, -5, 8, 8, None, 0, None) == -2
+    cfg = _lib.TileConfig()
+    assert lib.ffnk_tile_config(0, 1, 1, 1, None) == -1
+    # M == 0 is a valid no-op that touches no pointer
+    assert lib.ffnk_masked_linear_fwd(None, 8, None, None, 1, 8, None, None, 8, 0, 8, 8, None, 0, None) == 0
+
+
+def test_ops_validate_inputs():
+    x = torch.zeros(4, 8, dtype=torch.bfloat16)
+    w = torch.zeros(8, 8, dtype=torch.bfloat16)
+    m = torch.zeros(4, dtype=torch.bool)
+    with pytest.raises(ValueError, match="GPU"):
+        MaskedLinear.apply(x, w.T, w.T, m)
+    with pytest.raises(ValueError, match="bfloat16"):
+        MaskedLinear.apply(x.float(), w.T, w.T, m)
+    with pytest.raises(ValueError, match="2-D"):
+        MaskedLinear.apply(x[None], w.T, w.T, m)
+    with pytest.raises(ValueError):
+        MaskedFFN.apply(x, w.T, w.T, w.T, w.T, w.T, w.T, m)
+
+
+def test_workloads_are_seeded_and_shaped():
+    a, b = wl.cfg1_linear_fwd(0), wl.cfg1_linear_fwd(0)
+    assert torch.equal(a.x, b.x) and torch.equal(a.mask, b.mask) and torch.equal(a.Wv, b.Wv)
+    assert a.x.shape == (2048, 1024) and a.mask.sum().item() == 2 * wl.IMAGE_TOKENS
+    assert not torch.equal(a.x, wl.cfg1_linear_fwd(1).x)
+    m4 = wl.cfg4_mask(0)
+    per_seq = m4.sum(1).tolist()
+    assert set(per_seq) == {0, 2 * 576, 5 * 576, 4096}
+    c3 = wl.cfg3_linear_bwd()
+    assert c3.grad.shape == (8192, 1024) and 0.45 < c3.mask.float().mean() < 0.55
+    c5 = wl.cfg5_ffn_decode(1, "visual", d=64, h=128)
+    assert c5.algorithmic_bytes() == 3 * 64 * 128 * 2 + 2 * 64 * 2 + 1
+    c5b = wl.cfg5_ffn_decode(8, "bernoulli", d=64, h=128)
+    nv = int(c5b.mask.sum())
+    assert c5b.algorithmic_bytes() == 3 * 64 * 128 * 2 * (int(nv > 0) + int(nv < 8)) + 2 * 8 * 64 * 2 + 8
+    assert wl.cfg2_ffn_fwd().routed_flops == 2 * 8192 * 1024 * 2048 * 3

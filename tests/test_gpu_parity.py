@@ -13,7 +13,7 @@ from ffn_kernel_amd import MaskedFFN, MaskedLinear, _lib
 from ffn_kernel_amd import workloads as wl
 from oracle import cref
 from oracle import modules as om
-from helpers import assert_close, note
+from helpers import assert_close, assert_close_bf16_pair, note
 
 pytestmark = pytest.mark.gpu
 
@@ -89,7 +89,7 @@ def test_linear_fwd_vs_oracle(dev, M, K, N, p):
     assert_close(y, ref, f"linear fwd {M}x{K}x{N}")
     # and against the reference's own (blend-form, bf16) PyTorch module maths
     blend = om.linear_blend(w.x, w.Wv, w.Wt, w.mask)
-    assert_close(y, blend.double(), "vs blend-form bf16 module")
+    assert_close_bf16_pair(y, blend, "vs blend-form bf16 module")
 
 
 def test_linear_row_selection_is_exact(dev):
@@ -188,7 +188,7 @@ def test_ffn_fwd_vs_oracle(dev, M, d, h, p):
     torch.cuda.synchronize()
     assert out.dtype == torch.bfloat16 and out.shape == (M, d)
     assert_close(out, cref.ffn_fwd(w.x, w.W, w.mask), f"ffn {M}x{d}x{h}")
-    assert_close(out, om.ffn_blend(w.x, w.W, w.mask).double(), "vs blend-form bf16 module")
+    assert_close_bf16_pair(out, om.ffn_blend(w.x, w.W, w.mask), "vs blend-form bf16 module")
 
 
 def test_ffn_cfg2(dev):
