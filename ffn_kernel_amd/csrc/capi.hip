@@ -88,6 +88,15 @@ BwdPlan plan_bwd(int64_t M, int64_t K, int64_t N, bool dw_k_contig) {
   return p;
 }
 
+// The direct global->LDS path addresses operands with 32-bit byte offsets: from the start of A
+// when its rows are gathered, from the tile's first row otherwise (at most 256 rows away).
+bool direct_ok(int64_t K, int64_t gathered_rows, int64_t lda, int64_t ldb) {
+  constexpr int64_t k4g = (int64_t)1 << 32;
+  if (K <= 0 || K % 32 != 0) return false;
+  if (gathered_rows > 0 && gathered_rows * lda * 2 >= k4g) return false;
+  return 256 * lda * 2 < k4g && 256 * ldb * 2 < k4g;
+}
+
 bool use_stream_path(int64_t M) { return false && M <= kStreamMaxM; }
 
 }  // namespace
@@ -154,7 +163,9 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->lds_stages = 2;
   out->group_m = 8;
   out->split_k = splits;
-  out->direct_lds = (contraction % 64 == 0) ? 1 : 0;
+  out->direct_lds = (contraction > 0 && contraction % 32 == 0) ? 1 : 0;
+  out->block_k = out->direct_lds ? 32 : 64;
+  out->lds_stages = out->direct_lds ? 4 : 2;
   return FFNK_OK;
 }
 
@@ -192,7 +203,7 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
   g.C = y; g.ldc = y_stride_m;
   g.perm = r.perm; g.counts = r.counts;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
-  FFNK_HIP(launch_linear_gemm(pick_routed_tile(M, N, false), K % 64 == 0, g, stream), "linear GEMM");
+  FFNK_HIP(launch_linear_gemm(pick_routed_tile(M, N, false), direct_ok(K, M, x_stride_m, w_stride_n), g, stream), "linear GEMM");
   return FFNK_OK;
 }
 
@@ -264,7 +275,7 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
   up.C = H; up.ldc = ldh;
   up.perm = r.perm; up.counts = r.counts;
   up.M = (int)M; up.N = (int)h; up.K = (int)d;
-  FFNK_HIP(launch_up_gemm(pick_routed_tile(M, h, true), d % 64 == 0, up, stream), "up-projection GEMM");
+  FFNK_HIP(launch_up_gemm(pick_routed_tile(M, h, true), direct_ok(d, M, x_stride_m, up_stride_n), up, stream), "up-projection GEMM");
   FFNK_HIP(mark(1), "event record");
   GemmArgs dn;
   dn.A = H; dn.lda = ldh;
@@ -272,7 +283,7 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
   dn.C = out; dn.ldc = out_stride_m;
   dn.perm = r.perm; dn.counts = r.counts;
   dn.M = (int)M; dn.N = (int)d; dn.K = (int)h;
-  FFNK_HIP(launch_down_gemm(pick_routed_tile(M, d, false), h % 64 == 0, dn, stream), "down-projection GEMM");
+  FFNK_HIP(launch_down_gemm(pick_routed_tile(M, d, false), direct_ok(h, 0, ldh, down_stride_n), dn, stream), "down-projection GEMM");
   FFNK_HIP(mark(2), "event record");
   return FFNK_OK;
 }
@@ -293,7 +304,8 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   if (dx_stride_m < K) return fail(FFNK_E_STRIDE, "dx_stride_m=%lld < K=%lld", (long long)dx_stride_m, (long long)K);
 
   const bool fast = M > 0 && N > 0 && K % 8 == 0 && N % 8 == 0 && g_stride_m % 8 == 0 && g_stride_m >= N &&
-                    x_stride_m % 8 == 0 && x_stride_m >= K && aligned16(g) && aligned16(x);
+                    x_stride_m % 8 == 0 && x_stride_m >= K && aligned16(g) && aligned16(x) &&
+                    direct_ok(64, 0, padded_rows(M), padded_rows(M));  // transposed operands have M-long rows
   if (!fast) {
     GenericBwdArgs a;
     a.g = g; a.sgm = g_stride_m; a.x = x; a.sxm = x_stride_m;
@@ -329,7 +341,7 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   a.C = dx; a.ldc = dx_stride_m;
   a.perm = r.perm; a.counts = r.counts;
   a.M = (int)M; a.N = (int)K; a.K = (int)N;
-  FFNK_HIP(launch_linear_gemm(pick_routed_tile(M, K, false), N % 64 == 0, a, stream), "dx GEMM");
+  FFNK_HIP(launch_linear_gemm(pick_routed_tile(M, K, false), direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
 
   // ---- dW_g = x_g^T g_g, contraction over the rows of group g ----
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]

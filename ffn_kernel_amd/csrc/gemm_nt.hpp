@@ -6,9 +6,9 @@
 // on every mixed tile.
 //
 // Data path per workgroup: 64-column K slabs of the A and B panels go global -> LDS (directly,
-// bypassing registers, or staged through registers when K has a tail), double-buffered with
-// one barrier per slab; wavefronts read 16-byte MFMA fragments from an XOR-swizzled LDS
-// layout and issue v_mfma_f32_32x32x16_bf16.
+// bypassing registers, through a 4-stage ring of 32-column half-slabs; or staged through
+// registers in 64-column slabs when K is not a multiple of 32); wavefronts read 16-byte MFMA
+// fragments from an XOR-swizzled LDS layout and issue v_mfma_f32_32x32x16_bf16.
 #pragma once
 #include "common.hpp"
 #include "gemm_args.hpp"
@@ -19,16 +19,28 @@ constexpr int kBK = 64;          // K elements per LDS stage
 constexpr int kRowBytes = 128;   // kBK * sizeof(bf16)
 constexpr int kXcds = 8;         // MI355X: 8 XCDs, workgroups are dealt to them round-robin
 
-// LDS byte offset of 16-byte chunk c (0..7) of tile row r.  Two rows share a 256-byte line;
-// the chunk index is XORed with the row so that the 16 lanes of one ds_read_b128 phase
-// (16 consecutive rows, same logical chunk) hit 16 distinct 16-byte bank groups, and any
-// aligned 8 of them hit 8 distinct groups modulo 128 bytes.
-__host__ __device__ constexpr uint32_t lds_swizzle(uint32_t r, uint32_t c) {
+// ---------------------------------------------------------------------------------------------
+// LDS layouts.  Both keep every ds_read_b128 of an MFMA fragment (16 consecutive tile rows, same
+// logical 16-byte chunk, per 16-lane phase) on 16 distinct 16-byte bank groups, and let a
+// wavefront fill LDS in lane order (lane -> 16 bytes at lane * 16), which is what a
+// global->LDS load requires.
+//
+//  * "slab" layout, 128-byte rows (64 K elements): used by the register-staged path.
+//  * "half-slab" layout, 64-byte rows (32 K elements): used by the direct global->LDS ring.
+// ---------------------------------------------------------------------------------------------
+__host__ __device__ constexpr uint32_t lds_swizzle(uint32_t r, uint32_t c) {  // c in 0..7
   return ((r >> 1) << 8) | (((((r & 1u) ^ ((r >> 3) & 1u)) << 3) | (c ^ (r & 7u))) << 4);
+}
+__host__ __device__ constexpr uint32_t lds_swizzle_h(uint32_t r, uint32_t c) {  // c in 0..3
+  return ((r >> 2) << 8) | (((4u * (r & 3u)) + (c ^ ((r >> 2) & 3u))) << 4);
 }
 
 #define FFNK_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define FFNK_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+constexpr int kBKH = 32;        // K elements per ring stage
+constexpr int kRowBytesH = 64;  // kBKH * sizeof(bf16)
+constexpr int kStages = 4;      // ring depth: one stage computing, one landed, two in flight
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool DUAL_, bool GATHER_A_, bool SCATTER_C_,
           bool DIRECT_, int GROUP_M_>
@@ -40,7 +52,7 @@ struct RoutedGemmCfg {
   static constexpr bool DUAL = DUAL_;
   static constexpr bool GATHER_A = GATHER_A_;
   static constexpr bool SCATTER_C = SCATTER_C_;
-  static constexpr bool DIRECT = DIRECT_;   // global->LDS loads bypass registers (needs K % 64 == 0)
+  static constexpr bool DIRECT = DIRECT_;   // global->LDS loads bypass registers (needs K % 32 == 0)
   static constexpr int GROUP_M = GROUP_M_;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int NT = NWAVES * kWave;
@@ -50,16 +62,199 @@ struct RoutedGemmCfg {
   static constexpr int TM = WTM / 32;                      // 32x32 MFMA tiles per wave, M direction
   static constexpr int TN_OUT = WTN_OUT / 32;
   static constexpr int TN = DUAL ? 2 * TN_OUT : TN_OUT;    // accumulator tiles per wave, N direction
-  static constexpr int A_BYTES = BM * kRowBytes;
-  static constexpr int B_BYTES = BN * kRowBytes;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int A_BYTES = BM * kRowBytes;           // slab layout
+  static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
+  static constexpr int A_BYTES_H = BM * kRowBytesH;        // half-slab layout
+  static constexpr int STAGE_BYTES_H = (BM + BN) * kRowBytesH;
+  static constexpr int LDS_BYTES = DIRECT ? kStages * STAGE_BYTES_H : 2 * STAGE_BYTES;
   static_assert(WTM % 32 == 0 && WTN_OUT % 32 == 0, "wave tile must be a multiple of 32x32");
-  static_assert(NWAVES % 2 == 0, "direct loads need an even wave count");
-  static_assert((BM / 8) % NWAVES == 0 && (BN / 8) % NWAVES == 0, "panel rows must split evenly over waves");
+  static_assert(NWAVES % 2 == 0, "lane mapping of the slab layout needs an even wave count");
+  static_assert((BM / 16) % NWAVES == 0 && (BN / 16) % NWAVES == 0, "panel rows must split evenly over waves");
+  static_assert(!DUAL || (BN / 2) % 16 == 0, "gate/up split must fall on a 16-row load group");
 };
 
-// Per-thread description of which 16-byte chunks of the A and B panels this lane moves, and
-// which LDS fragments it reads.  Built once per tile by the kernels below.
+// Accumulator tile b of the wave reads B-panel rows starting here.
+template <class Cfg>
+__device__ __forceinline__ int b_frag_row(int wn, int tn) {
+  if (Cfg::DUAL) return (tn < Cfg::TN_OUT ? 0 : Cfg::BN / 2) + wn * Cfg::WTN_OUT + (tn % Cfg::TN_OUT) * 32;
+  return wn * Cfg::WTN_OUT + tn * 32;
+}
+
+template <class Cfg>
+__device__ __forceinline__ void zero_acc(f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
+#pragma unroll
+  for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+}
+
+// =============================================================================================
+// Direct path: 4-stage ring of 32-element K half-slabs, filled by buffer_load ... lds.
+// =============================================================================================
+// Which 16-byte chunks this lane moves.  A panel is moved as 1 KB groups of 16 rows x 64 bytes;
+// group id = j * NWAVES + wave; the lane fills physical slot `lane` of its group:
+//   lds_swizzle_h(group * 16 + r_in, c_log) == group * 1024 + lane * 16.
+template <class Cfg>
+struct RingLanes {
+  static constexpr int NJA = Cfg::BM / 16 / Cfg::NWAVES;
+  static constexpr int NJB = Cfg::BN / 16 / Cfg::NWAVES;
+  int lane, wave, wm, wn;
+  uint32_t r_in, c_log, lr, lh;
+  __device__ __forceinline__ void init() {
+    const int tid = threadIdx.x;
+    lane = tid & (kWave - 1);
+    wave = tid / kWave;
+    wm = wave / Cfg::WAVES_N;
+    wn = wave % Cfg::WAVES_N;
+    const uint32_t line = lane >> 4, slot = lane & 15;
+    r_in = 4 * line + (slot >> 2);
+    c_log = (slot & 3) ^ (line & 3);
+    lr = lane & 31;
+    lh = lane >> 5;
+  }
+  // First tile row of load group j of this wave (uniform over the wave), and this lane's row.
+  __device__ __forceinline__ int group_row(int j) const { return (j * Cfg::NWAVES + wave) * 16; }
+  __device__ __forceinline__ int load_row(int j) const { return group_row(j) + (int)r_in; }
+};
+
+constexpr int waitcnt_imm(int vm, int lgkm) {  // gfx9 s_waitcnt encoding, expcnt untouched
+  return (vm & 15) | (7 << 4) | ((lgkm & 15) << 8) | ((vm >> 4) << 14);
+}
+
+// Wait until at most N of this wave's global->LDS loads are outstanding and all of its LDS reads
+// have returned, then barrier.  Written with builtins (not a fence) so that younger loads stay
+// in flight across the barrier.
+template <int N>
+__device__ __forceinline__ void ring_wait_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(N, 0));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// K loop of one tile on the ring.  Load j of the A panel reads 16 bytes at baseA[j] + offA[j]
+// (+ 64 bytes per half-slab); baseA[j] is uniform over the wave, offA[j] is this lane's 32-bit
+// byte offset.  Likewise for B.  k_len is a positive multiple of 32.
+//
+// Iteration i: [wait: half-slab i+1 landed everywhere, stage of i-1 free] [issue loads of i+3]
+// then the MFMAs of half-slab i, whose first fragments were read during iteration i-1, with
+// the LDS reads of its second K step, the reads of the first fragments of half-slab i+1 and
+// the global->LDS loads interleaved one per MFMA, so that the matrix pipe never waits for a
+// barrier or an LDS round trip.
+template <class Cfg>
+__device__ __forceinline__ void gemm_mainloop_ring(const RingLanes<Cfg>& rl,
+                                                   const uint16_t* const (&baseA)[RingLanes<Cfg>::NJA],
+                                                   const uint32_t (&offA)[RingLanes<Cfg>::NJA],
+                                                   const uint16_t* const (&baseB)[RingLanes<Cfg>::NJB],
+                                                   const uint32_t (&offB)[RingLanes<Cfg>::NJB], int k_len,
+                                                   uint8_t* lds, f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
+  constexpr int NJA = RingLanes<Cfg>::NJA, NJB = RingLanes<Cfg>::NJB;
+  constexpr int L = NJA + NJB;  // loads per wave per half-slab
+  constexpr int NS = kStages;
+  constexpr int STAGE = Cfg::STAGE_BYTES_H, A_BYTES = Cfg::A_BYTES_H;
+  constexpr int NM = TM * TN, ND = TM + TN;
+  const int wave = rl.wave;
+
+  __amdgpu_buffer_rsrc_t rsA[NJA], rsB[NJB];
+#pragma unroll
+  for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc((void*)baseA[j], 0, 0xffffffff, 0x00020000);
+#pragma unroll
+  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc((void*)baseB[j], 0, 0xffffffff, 0x00020000);
+
+  uint32_t koff[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) koff[s] = lds_swizzle_h(rl.lr, 2 * s + rl.lh);
+  const uint32_t a_base = (uint32_t)(rl.wm * Cfg::WTM) * kRowBytesH;
+  uint32_t b_base[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) b_base[tn] = A_BYTES + (uint32_t)b_frag_row<Cfg>(rl.wn, tn) * kRowBytesH;
+
+  zero_acc<Cfg>(acc);
+  const int nh = k_len / kBKH;
+
+  auto issue = [&](int stage, int ih) {
+    uint8_t* st = lds + stage * STAGE;
+    const int kb = ih * kRowBytesH;
+#pragma unroll
+    for (int j = 0; j < NJA; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[j], FFNK_LDS_PTR(st + (j * NWAVES + wave) * 1024), 16, offA[j], kb, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NJB; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[j], FFNK_LDS_PTR(st + A_BYTES + (j * NWAVES + wave) * 1024), 16, offB[j], kb, 0, 0);
+  };
+  bf16x8_t fa[2][TM], fb[2][TN];
+  auto load_frags = [&](int buf, int stage, int s) {
+    const uint8_t* st = lds + stage * STAGE;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      fa[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_base + i * 32 * kRowBytesH + koff[s]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_base[j] + koff[s]);
+  };
+  auto mfmas = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        // D[n][m]: the weights are the MFMA "A" operand, so each lane ends up with runs of four
+        // consecutive output columns of one token row.
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+  };
+
+  // Prologue: fill NS-1 stages, wait for the first, read its first fragments.
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s)
+    if (s < nh) issue(s, s);
+  if (nh > NS - 2) ring_wait_barrier<(NS - 2) * L>();
+  else ring_wait_barrier<0>();
+  load_frags(0, 0, 0);
+
+  auto body = [&](int u, int i, bool full) {
+    if (full || i + NS - 2 < nh) ring_wait_barrier<(NS - 3) * L>();
+    else ring_wait_barrier<0>();
+    if (full || i + NS - 1 < nh) issue((u + NS - 1) % NS, i + NS - 1);
+    load_frags(1, u, 1);
+    mfmas(0);
+    if (full || i + 1 < nh) load_frags(0, (u + 1) % NS, 0);
+    mfmas(1);
+    if (full) {
+      // Issue order inside the (branch-free) steady-state iteration: one LDS read after each of
+      // the first TM+TN MFMAs of a K step, one global->LDS load after each of the next ones.
+#pragma unroll
+      for (int q = 0; q < NM; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (q < ND) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        else if (q - ND < L) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+#pragma unroll
+      for (int q = 0; q < NM; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (q < ND) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        else if (q - ND + (NM - ND) < L) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+    }
+  };
+  int i0 = 0;
+  for (; i0 + 2 * NS - 2 < nh; i0 += NS) {  // every guard inside is true: no branches
+#pragma unroll
+    for (int u = 0; u < NS; ++u) body(u, i0 + u, true);
+  }
+  for (; i0 < nh; i0 += NS) {
+#pragma unroll
+    for (int u = 0; u < NS; ++u)
+      if (i0 + u < nh) body(u, i0 + u, false);
+  }
+#endif
+}
+
+// =============================================================================================
+// Register-staged path: 64-element K slabs, global -> registers -> LDS, double-buffered.  Handles
+// any K that is a multiple of 8 (chunks past the end are zero-filled).
+// =============================================================================================
 template <class Cfg>
 struct TileLanes {
   static constexpr int NJA = Cfg::BM / 8 / Cfg::NWAVES;  // 1 KB (8-row) groups of the A panel per wave
@@ -75,70 +270,41 @@ struct TileLanes {
     wave = tid / kWave;
     wm = wave / Cfg::WAVES_N;
     wn = wave % Cfg::WAVES_N;
-    // The panel is moved as 1 KB groups of 8 rows; group id = j * NWAVES + wave, so the group's
-    // parity (which the swizzle needs) is the wave's parity.  The lane fills physical 16-byte
-    // slot `lane` of the group: lds_swizzle(group * 8 + r_in, c_log) == group * 1024 + lane * 16.
+    // Group id = j * NWAVES + wave, so the group's parity (which the swizzle needs) is the wave's
+    // parity.  lds_swizzle(group * 8 + r_in, c_log) == group * 1024 + lane * 16.
     const uint32_t q = lane & 15;
     r_in = 2 * (lane >> 4) + ((q >> 3) ^ (wave & 1));
     c_log = (q & 7) ^ r_in;
     lr = lane & 31;
     lh = lane >> 5;
   }
-  // Tile row that load j of this lane covers.
   __device__ __forceinline__ int load_row(int j) const { return (j * Cfg::NWAVES + wave) * 8 + (int)r_in; }
 };
 
-// K loop of one tile.  pa[j] / pb[j] point at this lane's chunk of slab 0 for each of its rows;
-// `k_len` is the contraction length from there (a multiple of 8; of 64 when Cfg::DIRECT).
-// Accumulates into acc[TM][TN] (32x32 tiles, D[n][m] orientation: the weights are the MFMA "A"
-// operand so that each lane ends up with runs of four consecutive output columns of one token row).
+// pa[j] / pb[j] point at this lane's chunk of slab 0 for each of its rows; k_len % 8 == 0.
 template <class Cfg>
-__device__ __forceinline__ void gemm_mainloop(const TileLanes<Cfg>& tl,
-                                              const uint16_t* const (&pa)[TileLanes<Cfg>::NJA],
-                                              const uint16_t* const (&pb)[TileLanes<Cfg>::NJB], int k_len,
-                                              uint8_t* lds0, uint8_t* lds1,
-                                              f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
-  constexpr int BN = Cfg::BN, NWAVES = Cfg::NWAVES;
-  constexpr int TM = Cfg::TM, TN = Cfg::TN, TN_OUT = Cfg::TN_OUT;
+__device__ __forceinline__ void gemm_mainloop_staged(const TileLanes<Cfg>& tl,
+                                                     const uint16_t* const (&pa)[TileLanes<Cfg>::NJA],
+                                                     const uint16_t* const (&pb)[TileLanes<Cfg>::NJB], int k_len,
+                                                     uint8_t* lds, f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
+  constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
   constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
   const int lane = tl.lane, wave = tl.wave;
+  uint8_t* lds0 = lds;
+  uint8_t* lds1 = lds + Cfg::STAGE_BYTES;
 
-  // Fragment rows start at multiples of 32, so the swizzle terms depend on the lane only.
   uint32_t koff[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) koff[s] = lds_swizzle(tl.lr, 2 * s + tl.lh);
   const uint32_t a_base = (uint32_t)(tl.wm * Cfg::WTM) * kRowBytes;
   uint32_t b_base[TN];
 #pragma unroll
-  for (int tn = 0; tn < TN; ++tn) {
-    int r;
-    if (Cfg::DUAL) r = (tn < TN_OUT ? 0 : BN / 2) + tl.wn * Cfg::WTN_OUT + (tn % TN_OUT) * 32;
-    else r = tl.wn * Cfg::WTN_OUT + tn * 32;
-    b_base[tn] = Cfg::A_BYTES + (uint32_t)r * kRowBytes;
-  }
+  for (int tn = 0; tn < TN; ++tn) b_base[tn] = Cfg::A_BYTES + (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
 
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
+  zero_acc<Cfg>(acc);
   const int nk = cdiv(k_len, kBK);
 
-  auto issue_direct = [&](uint8_t* stage, int kt) {
-    const int64_t ko = (int64_t)kt * kBK;
-#pragma unroll
-    for (int j = 0; j < NJA; ++j)
-      __builtin_amdgcn_global_load_lds(FFNK_GLOBAL_PTR(pa[j] + ko),
-                                       FFNK_LDS_PTR(stage + (j * NWAVES + wave) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int j = 0; j < NJB; ++j)
-      __builtin_amdgcn_global_load_lds(FFNK_GLOBAL_PTR(pb[j] + ko),
-                                       FFNK_LDS_PTR(stage + Cfg::A_BYTES + (j * NWAVES + wave) * 1024), 16, 0, 0);
-  };
-
-  uint4 ra[NJA], rb[NJB];  // register staging (only live when !DIRECT)
+  uint4 ra[NJA], rb[NJB];
   auto load_regs = [&](int kt) {
     // k_len % 8 == 0, so a 16-byte chunk is entirely inside or entirely outside the tail.
     const bool ok = kt * kBK + (int)tl.c_log * 8 + 8 <= k_len;
@@ -158,7 +324,6 @@ __device__ __forceinline__ void gemm_mainloop(const TileLanes<Cfg>& tl,
     for (int j = 0; j < NJB; ++j)
       *reinterpret_cast<uint4*>(stage + Cfg::A_BYTES + (j * NWAVES + wave) * 1024 + lane * 16) = rb[j];
   };
-
   auto compute = [&](const uint8_t* stage) {
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -178,32 +343,18 @@ __device__ __forceinline__ void gemm_mainloop(const TileLanes<Cfg>& tl,
   };
 
   if (nk <= 0) return;
-  if (Cfg::DIRECT) {
-    issue_direct(lds0, 0);
-    for (int kt = 0; kt < nk; kt += 2) {
-      __syncthreads();  // slab kt has landed everywhere; everyone is done reading lds1
-      if (kt + 1 < nk) issue_direct(lds1, kt + 1);
-      compute(lds0);
-      if (kt + 1 < nk) {
-        __syncthreads();
-        if (kt + 2 < nk) issue_direct(lds0, kt + 2);
-        compute(lds1);
-      }
-    }
-  } else {
-    load_regs(0);
-    store_regs(lds0);
-    for (int kt = 0; kt < nk; kt += 2) {
+  load_regs(0);
+  store_regs(lds0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    __syncthreads();
+    if (kt + 1 < nk) load_regs(kt + 1);
+    compute(lds0);
+    if (kt + 1 < nk) {
+      store_regs(lds1);
       __syncthreads();
-      if (kt + 1 < nk) load_regs(kt + 1);
-      compute(lds0);
-      if (kt + 1 < nk) {
-        store_regs(lds1);
-        __syncthreads();
-        if (kt + 2 < nk) load_regs(kt + 2);
-        compute(lds1);
-        if (kt + 2 < nk) store_regs(lds0);
-      }
+      if (kt + 2 < nk) load_regs(kt + 2);
+      compute(lds1);
+      if (kt + 2 < nk) store_regs(lds0);
     }
   }
 }
@@ -219,81 +370,21 @@ __device__ __forceinline__ int xcd_tile_slot(int total) {
   return L < total ? L : -1;
 }
 
-// Routed GEMM: rows in routed order, group-pure tiles.
-//   GATHER_A : A row of routed position p is perm[p] (else p)
-//   SCATTER_C: C row of routed position p is perm[p] (else p)
-//   DUAL     : C = silu(A B0^T) * (A B1^T)   (SwiGLU epilogue in fp32 registers)
+// Epilogue shared by the routed kernels.  Per 32x32 accumulator tile a lane holds token row
+// (lane & 31) and output columns 8 * (v / 4) + 4 * (lane >> 5) + (v % 4).
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) {
-  constexpr int BM = Cfg::BM, BN = Cfg::BN;
-  constexpr int TM = Cfg::TM, TN = Cfg::TN, TN_OUT = Cfg::TN_OUT;
-  constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
-
-  __shared__ __attribute__((aligned(1024))) uint8_t lds0[Cfg::STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t lds1[Cfg::STAGE_BYTES];
-
-  // ---- tile schedule (all from device-side counts; no host sync) ----
-  const int n_vis = g.counts[0];
-  const int n_txt = g.M - n_vis;
-  const int tiles_v = cdiv(n_vis, BM);
-  const int tiles_m = tiles_v + cdiv(n_txt, BM);
-  const int tiles_n = cdiv(g.N, Cfg::BN_OUT);
-  const int L = xcd_tile_slot(tiles_m * tiles_n);
-  if (L < 0) return;
-  const int width = Cfg::GROUP_M * tiles_n;
-  const int first_m = (L / width) * Cfg::GROUP_M;
-  const int gsz = min(Cfg::GROUP_M, tiles_m - first_m);
-  const int tile_m = first_m + (L % width) % gsz;
-  const int tile_n = (L % width) / gsz;
-
-  const int grp = tile_m < tiles_v ? 0 : 1;
-  const int row0 = grp == 0 ? tile_m * BM : n_vis + (tile_m - tiles_v) * BM;  // routed position
-  const int row_end = grp == 0 ? n_vis : g.M;
-  const int n0 = tile_n * Cfg::BN_OUT;
-
-  TileLanes<Cfg> tl;
-  tl.init();
-
-  const uint16_t* pa[NJA];
-  const uint16_t* pb[NJB];
-#pragma unroll
-  for (int j = 0; j < NJA; ++j) {
-    int p = row0 + tl.load_row(j);
-    p = min(p, row_end - 1);  // rows past the group end repeat the last row; never stored
-    const int64_t src = Cfg::GATHER_A ? (int64_t)g.perm[p] : (int64_t)p;
-    pa[j] = g.A + src * g.lda + tl.c_log * 8;
-  }
-#pragma unroll
-  for (int j = 0; j < NJB; ++j) {
-    const int r = tl.load_row(j);  // row of the LDS B panel
-    const uint16_t* base;
-    int n;
-    if (Cfg::DUAL) {
-      const bool up = r >= BN / 2;
-      base = up ? g.B1[grp] : g.B0[grp];
-      n = n0 + (up ? r - BN / 2 : r);
-    } else {
-      base = g.B0[grp];
-      n = n0 + r;
-    }
-    n = min(n, g.N - 1);
-    pb[j] = base + (int64_t)n * g.ldb + tl.c_log * 8;
-  }
-
-  f32x16_t acc[TM][TN];
-  gemm_mainloop<Cfg>(tl, pa, pb, g.K, lds0, lds1, acc);
-
-  // ---- epilogue: lane holds, per 32x32 tile, token row (lane & 31) and output columns
-  //      8 * (v / 4) + 4 * (lane >> 5) + (v % 4) ----
+__device__ __forceinline__ void routed_epilogue(const GemmArgs& g, f32x16_t (&acc)[Cfg::TM][Cfg::TN], int row0,
+                                                int row_end, int n0, int wm, int wn, uint32_t lr, uint32_t lh) {
+  constexpr int TM = Cfg::TM, TN_OUT = Cfg::TN_OUT;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int p = row0 + tl.wm * Cfg::WTM + i * 32 + (int)tl.lr;
+    const int p = row0 + wm * Cfg::WTM + i * 32 + (int)lr;
     if (p >= row_end) continue;
     const int64_t dst = Cfg::SCATTER_C ? (int64_t)g.perm[p] : (int64_t)p;
     uint16_t* crow = g.C + dst * g.ldc;
 #pragma unroll
     for (int j = 0; j < TN_OUT; ++j) {
-      const int nb = n0 + tl.wn * Cfg::WTN_OUT + j * 32 + 4 * (int)tl.lh;
+      const int nb = n0 + wn * Cfg::WTN_OUT + j * 32 + 4 * (int)lh;
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         const int n = nb + 8 * q4;
@@ -318,15 +409,102 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   }
 }
 
+// Routed GEMM: rows in routed order, group-pure tiles.
+//   GATHER_A : A row of routed position p is perm[p] (else p)
+//   SCATTER_C: C row of routed position p is perm[p] (else p)
+//   DUAL     : C = silu(A B0^T) * (A B1^T)   (SwiGLU epilogue in fp32 registers)
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN;
+
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[Cfg::LDS_BYTES];
+
+  // ---- tile schedule (all from device-side counts; no host sync) ----
+  const int n_vis = g.counts[0];
+  const int n_txt = g.M - n_vis;
+  const int tiles_v = cdiv(n_vis, BM);
+  const int tiles_m = tiles_v + cdiv(n_txt, BM);
+  const int tiles_n = cdiv(g.N, Cfg::BN_OUT);
+  const int L = xcd_tile_slot(tiles_m * tiles_n);
+  if (L < 0) return;
+  const int width = Cfg::GROUP_M * tiles_n;
+  const int first_m = (L / width) * Cfg::GROUP_M;
+  const int gsz = min(Cfg::GROUP_M, tiles_m - first_m);
+  const int tile_m = first_m + (L % width) % gsz;
+  const int tile_n = (L % width) / gsz;
+
+  const int grp = tile_m < tiles_v ? 0 : 1;
+  const int row0 = grp == 0 ? tile_m * BM : n_vis + (tile_m - tiles_v) * BM;  // routed position
+  const int row_end = grp == 0 ? n_vis : g.M;
+  const int n0 = tile_n * Cfg::BN_OUT;
+
+  f32x16_t acc[TM][TN];
+  if (Cfg::DIRECT) {
+    constexpr int NJA = RingLanes<Cfg>::NJA, NJB = RingLanes<Cfg>::NJB;
+    RingLanes<Cfg> rl;
+    rl.init();
+    const uint16_t* baseA[NJA];
+    uint32_t offA[NJA];
+    const uint16_t* baseB[NJB];
+    uint32_t offB[NJB];
+    // Gathered rows are addressed from the start of A (the host checks that 32 bits reach every
+    // row); contiguous panels from their own first row.
+    const uint16_t* a0 = Cfg::GATHER_A ? g.A : g.A + (int64_t)row0 * g.lda;
+#pragma unroll
+    for (int j = 0; j < NJA; ++j) {
+      int p = row0 + rl.load_row(j);
+      p = min(p, row_end - 1);  // rows past the group end repeat the last row; never stored
+      const int64_t src = Cfg::GATHER_A ? (int64_t)g.perm[p] : (int64_t)(p - row0);
+      baseA[j] = a0;
+      offA[j] = (uint32_t)((src * g.lda + rl.c_log * 8) * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < NJB; ++j) {
+      const bool up = Cfg::DUAL && rl.group_row(j) >= BN / 2;  // uniform over the wave
+      const int r = rl.load_row(j) - (up ? BN / 2 : 0);
+      const int n_first = min(n0, g.N - 1);
+      const int n = min(n0 + r, g.N - 1);
+      baseB[j] = (up ? g.B1[grp] : g.B0[grp]) + (int64_t)n_first * g.ldb;
+      offB[j] = (uint32_t)(((int64_t)(n - n_first) * g.ldb + rl.c_log * 8) * 2);
+    }
+    gemm_mainloop_ring<Cfg>(rl, baseA, offA, baseB, offB, g.K, lds, acc);
+    routed_epilogue<Cfg>(g, acc, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
+  } else {
+    constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
+    TileLanes<Cfg> tl;
+    tl.init();
+    const uint16_t* pa[NJA];
+    const uint16_t* pb[NJB];
+#pragma unroll
+    for (int j = 0; j < NJA; ++j) {
+      int p = row0 + tl.load_row(j);
+      p = min(p, row_end - 1);
+      const int64_t src = Cfg::GATHER_A ? (int64_t)g.perm[p] : (int64_t)p;
+      pa[j] = g.A + src * g.lda + tl.c_log * 8;
+    }
+#pragma unroll
+    for (int j = 0; j < NJB; ++j) {
+      const int r = tl.load_row(j);  // row of the LDS B panel
+      const bool up = Cfg::DUAL && r >= BN / 2;
+      const int n = min(n0 + (up ? r - BN / 2 : r), g.N - 1);
+      pb[j] = (up ? g.B1[grp] : g.B0[grp]) + (int64_t)n * g.ldb + tl.c_log * 8;
+    }
+    gemm_mainloop_staged<Cfg>(tl, pa, pb, g.K, lds, acc);
+    routed_epilogue<Cfg>(g, acc, row0, row_end, n0, tl.wm, tl.wn, tl.lr, tl.lh);
+  }
+}
+
+// Grouped split-K GEMM of the weight gradients (operands are padded to 64-element slabs, so
+// the ring path always applies).
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArgs g) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
-  constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
+  constexpr int NJA = RingLanes<Cfg>::NJA, NJB = RingLanes<Cfg>::NJB;
   static_assert(!Cfg::DUAL && Cfg::DIRECT, "split-K GEMM runs on padded, 64-aligned slabs");
 
-  __shared__ __attribute__((aligned(1024))) uint8_t lds0[Cfg::STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t lds1[Cfg::STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[Cfg::LDS_BYTES];
 
   // The BM-row LDS panel holds rows of B (output columns) and the BN-row panel holds rows of A
   // (output rows): a 32-lane half wave then owns 32 consecutive output columns of one output
@@ -353,46 +531,45 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
   const int64_t k_begin = (int64_t)k_begin_g + (int64_t)kt0 * kBK;
   const int k_len = (kt1 - kt0) * kBK;
 
-  TileLanes<Cfg> tl;
-  tl.init();
+  RingLanes<Cfg> rl;
+  rl.init();
   const int r0 = tile_r * BN, c0 = tile_c * BM;
-  const uint16_t* pa[NJA];
-  const uint16_t* pb[NJB];
-#pragma unroll
-  for (int j = 0; j < NJA; ++j) {
-    const int c = min(c0 + tl.load_row(j), g.Cc - 1);
-    pa[j] = g.B + (int64_t)c * g.ldb + k_begin + tl.c_log * 8;
-  }
-#pragma unroll
-  for (int j = 0; j < NJB; ++j) {
-    const int r = min(r0 + tl.load_row(j), g.R - 1);
-    pb[j] = g.A + (int64_t)r * g.lda + k_begin + tl.c_log * 8;
-  }
-
   f32x16_t acc[TM][TN];
   if (k_len > 0) {
-    gemm_mainloop<Cfg>(tl, pa, pb, k_len, lds0, lds1, acc);
+    const uint16_t* baseA[NJA];
+    uint32_t offA[NJA];
+    const uint16_t* baseB[NJB];
+    uint32_t offB[NJB];
+    const int c_first = min(c0, g.Cc - 1), r_first = min(r0, g.R - 1);
+#pragma unroll
+    for (int j = 0; j < NJA; ++j) {
+      const int c = min(c0 + rl.load_row(j), g.Cc - 1);
+      baseA[j] = g.B + (int64_t)c_first * g.ldb + k_begin;
+      offA[j] = (uint32_t)(((int64_t)(c - c_first) * g.ldb + rl.c_log * 8) * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < NJB; ++j) {
+      const int r = min(r0 + rl.load_row(j), g.R - 1);
+      baseB[j] = g.A + (int64_t)r_first * g.lda + k_begin;
+      offB[j] = (uint32_t)(((int64_t)(r - r_first) * g.lda + rl.c_log * 8) * 2);
+    }
+    gemm_mainloop_ring<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc);
   } else {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    zero_acc<Cfg>(acc);  // a split without slabs (e.g. an empty modality) contributes exact zeros
   }
 
-  // acc[i][j][v]: panel-"x" row (= output column c) c0 + wm*WTM + i*32 + (lane&31);
-  //               panel-"weight" row (= output row r) r0 + wn*WTN + j*32 + 8*(v/4) + 4*(lane>>5) + v%4.
+  // acc[i][j][v]: BM-panel row (= output column c) c0 + wm*WTM + i*32 + (lane&31);
+  //               BN-panel row (= output row r) r0 + wn*WTN + j*32 + 8*(v/4) + 4*(lane>>5) + v%4.
   float* P = g.P + ((int64_t)(grp * g.splits + split)) * g.R * g.Cc;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int c = c0 + tl.wm * Cfg::WTM + i * 32 + (int)tl.lr;
+    const int c = c0 + rl.wm * Cfg::WTM + i * 32 + (int)rl.lr;
     if (c >= g.Cc) continue;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int r = r0 + tl.wn * Cfg::WTN_OUT + j * 32 + 8 * (v / 4) + 4 * (int)tl.lh + (v % 4);
+        const int r = r0 + rl.wn * Cfg::WTN_OUT + j * 32 + 8 * (v / 4) + 4 * (int)rl.lh + (v % 4);
         if (r < g.R) P[(int64_t)r * g.Cc + c] = acc[i][j][v];  // 32 lanes -> 32 consecutive floats
       }
     }

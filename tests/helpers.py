@@ -24,9 +24,11 @@ def assert_close(got: torch.Tensor, ref: torch.Tensor, what: str) -> dict:
 def assert_close_bf16_pair(got: torch.Tensor, other_bf16: torch.Tensor, what: str) -> dict:
     """Two bf16 results of the same maths (e.g. the kernel and the reference's bf16 PyTorch modules,
     which round after every Linear / silu / product): each is within the bounds above of the exact
-    value, so they may differ from one another by twice those bounds (4e-2, 1e-2), and the module
-    form adds its intermediate roundings on top (measured up to ~6e-3 rel-L2 on tiny shapes)."""
+    value, so they may differ from one another by twice those bounds, and the module form adds its
+    intermediate roundings on top (four for the FFN: both projections, silu, product).  Bound used:
+    every element within 4x (2e-2 or one bf16 ulp), rel-L2 <= 1.5e-2.  This is a sanity check
+    against the reference's own formulation; the tight check is the one against the exact oracle."""
     rep = om.error_report(got.detach().float().cpu(), other_bf16.double())
-    ok = rep["max_excess"] <= 2.0 and rep["rel_l2"] <= 3 * om.REL_L2_TOL
+    ok = rep["max_excess"] <= 4.0 and rep["rel_l2"] <= 3 * om.REL_L2_TOL
     assert ok, f"{what}: {rep}"
     return rep
