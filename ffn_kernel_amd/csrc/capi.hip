@@ -97,7 +97,7 @@ bool direct_ok(int64_t K, int64_t gathered_rows, int64_t lda, int64_t ldb) {
   return 256 * lda * 2 < k4g && 256 * ldb * 2 < k4g;
 }
 
-bool use_stream_path(int64_t M) { return false && M <= kStreamMaxM; }
+bool use_stream_path(int64_t M, int64_t d, int64_t h) { return stream_shape_ok(M, d, h); }
 
 }  // namespace
 
@@ -120,8 +120,10 @@ size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
     case FFNK_OP_LINEAR_FWD:
       return route_ws_bytes(M);
     case FFNK_OP_FFN_FWD:
-      // perm + counts + the [M, h] bf16 intermediate in routed order (N = h).
-      return route_ws_bytes(M) + ws_align((size_t)M * round_up64(N, 8) * 2);
+      // perm + counts + the [M, h] bf16 intermediate in routed order (N = h); the streaming path
+      // adds the fp32 split-K partials of the down projection.
+      return route_ws_bytes(M) + ws_align((size_t)M * round_up64(N, 8) * 2) +
+             (use_stream_path(M, K, N) ? ws_align((size_t)stream_down_splits(K, N) * M * K * 4) : 0);
     case FFNK_OP_LINEAR_BWD: {
       const BwdPlan a = plan_bwd(M, K, N, true), b = plan_bwd(M, K, N, false);
       return a.total > b.total ? a.total : b.total;
@@ -153,7 +155,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
     default: return fail(FFNK_E_OP, "unknown op %d", op);
   }
   const TileGeom gm = tile_geom(tile, dual);
-  const bool stream = (op == FFNK_OP_FFN_FWD || op == FFNK_OP_FFN_UP || op == FFNK_OP_FFN_DOWN) && use_stream_path(M);
+  const bool stream = (op == FFNK_OP_FFN_FWD || op == FFNK_OP_FFN_UP || op == FFNK_OP_FFN_DOWN) && use_stream_path(M, K, N);
   out->path = stream ? FFNK_PATH_STREAM : FFNK_PATH_MFMA_TILED;
   out->block_m = gm.block_m;
   out->block_n = gm.block_n_out;
@@ -166,6 +168,20 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->direct_lds = (contraction > 0 && contraction % 32 == 0) ? 1 : 0;
   out->block_k = out->direct_lds ? 32 : 64;
   out->lds_stages = out->direct_lds ? 4 : 2;
+  if (stream) {
+    // Streaming kernels: a workgroup is 16 * RT weight rows x one K range whose four wavefronts
+    // take a quarter each; operands go global -> registers, no LDS staging.
+    const bool up = op != FFNK_OP_FFN_DOWN;
+    out->block_m = 16 * (int)cdiv64(M, 16);
+    out->block_n = stream_rows_per_block((int)M, up);
+    out->block_k = stream_chunk_k((int)M, up);
+    out->waves_m = 1;
+    out->waves_n = 1;
+    out->lds_stages = 0;
+    out->group_m = 1;
+    out->split_k = 4 * (up ? 1 : stream_down_splits(K, N));
+    out->direct_lds = 0;
+  }
   return FFNK_OK;
 }
 
@@ -263,6 +279,26 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
     a.mask = mask; a.y = out; a.sym = out_stride_m; a.syn = 1;
     a.M = (int)M; a.K = (int)h; a.N = (int)d;
     FFNK_HIP(launch_generic_linear(a, stream), "generic down kernel");
+    FFNK_HIP(mark(2), "event record");
+    return FFNK_OK;
+  }
+
+  if (use_stream_path(M, d, h)) {
+    float* P = reinterpret_cast<float*>(wsb + r.bytes + ws_align((size_t)M * ldh * 2));
+    const int splits = stream_down_splits(d, h);
+    FFNK_HIP(mark(0), "event record");
+    StreamArgs u;
+    u.X = x; u.ldx = x_stride_m; u.gather_x = 1; u.mask = mask; u.M = (int)M;
+    u.W0[0] = W1; u.W0[1] = U1; u.W1[0] = W3; u.W1[1] = U3; u.ldw = up_stride_n;
+    u.Nrows = (int)h; u.K = (int)d; u.splits = 1; u.H = H; u.ldh = ldh; u.P = nullptr;
+    FFNK_HIP(launch_stream_up(u, stream), "streaming up-projection");
+    FFNK_HIP(mark(1), "event record");
+    StreamArgs dn;
+    dn.X = H; dn.ldx = ldh; dn.gather_x = 0; dn.mask = mask; dn.M = (int)M;
+    dn.W0[0] = W2; dn.W0[1] = U2; dn.W1[0] = dn.W1[1] = nullptr; dn.ldw = down_stride_n;
+    dn.Nrows = (int)d; dn.K = (int)h; dn.splits = splits; dn.H = nullptr; dn.ldh = 0; dn.P = P;
+    FFNK_HIP(launch_stream_down(dn, stream), "streaming down-projection");
+    FFNK_HIP(launch_stream_reduce(P, splits, (int)M, (int)d, mask, out, out_stride_m, stream), "streaming reduce");
     FFNK_HIP(mark(2), "event record");
     return FFNK_OK;
   }

@@ -46,6 +46,27 @@ hipError_t launch_gather_transpose(const uint16_t* src, int64_t ld_src, const in
 hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint16_t* out0, uint16_t* out1,
                                 int64_t sr, int64_t sc, hipStream_t stream);
 
+// ---- stream.hip: weight-streaming kernels for M <= 64 ----
+struct StreamArgs {
+  const uint16_t* X; int64_t ldx;  // token rows: x [M, K] (gather_x = 1, token order) or H [M, K] (routed order)
+  int gather_x;
+  const uint8_t* mask; int M;      // M <= 64
+  const uint16_t* W0[2];           // per group: weight rows [Nrows, K], K contiguous
+  const uint16_t* W1[2];           // up-projection only: the second ("up") weight
+  int64_t ldw;
+  int Nrows, K, splits;            // K % 256 == 0; splits > 1 only for the down projection
+  uint16_t* H; int64_t ldh;        // up-projection output, routed order [M, Nrows]
+  float* P;                        // down-projection partials [splits][M][Nrows] (routed order)
+};
+// Shape of the streaming kernels for M rows (reported through ffnk_tile_config).
+int stream_rows_per_block(int M, bool dual);  // weight rows (of each matrix) per workgroup
+int stream_chunk_k(int M, bool dual);         // K elements per streamed chunk
+hipError_t launch_stream_up(const StreamArgs& a, hipStream_t stream);
+hipError_t launch_stream_down(const StreamArgs& a, hipStream_t stream);
+// out[token row of p, n] = bf16(sum_s P[s][p][n])
+hipError_t launch_stream_reduce(const float* P, int splits, int M, int N, const uint8_t* mask, uint16_t* out,
+                                int64_t ldo, hipStream_t stream);
+
 // ---- generic.hip: any-stride scalar kernels ----
 struct GenericLinearArgs {
   const uint16_t* x; int64_t sxm, sxk;

@@ -46,4 +46,25 @@ inline TileChoice pick_splitk_tile(int64_t M, int64_t R, int64_t Cc) {
   return c;
 }
 
+// Decode shapes: the streaming kernels need whole 128-element K chunks in both projections.
+inline bool stream_shape_ok(int64_t M, int64_t d, int64_t h) {
+  return M >= 1 && M <= kStreamMaxM && d >= 128 && h >= 128 && d % 128 == 0 && h % 128 == 0 && d % 16 == 0;
+}
+
+// Split-K factor of the streamed down-projection.  A workgroup covers 16 weight rows x one K
+// range (its four wavefronts take a quarter each); aim at about 16 wavefronts per CU and per
+// modality, keep at least four 128-element chunks per workgroup, and prefer a split that gives
+// every wavefront the same number of chunks.
+inline int stream_down_splits(int64_t d, int64_t h) {
+  const int64_t row_blocks = cdiv64(d, 16);
+  const int64_t chunks = h / 128;
+  int64_t s = cdiv64(4 * kCus, row_blocks);
+  if (s > chunks / 4) s = chunks / 4;
+  if (s > 16) s = 16;
+  if (s < 1) s = 1;
+  for (int64_t c = s; c >= 1 && c * 2 > s; --c)
+    if (chunks % (c * 4) == 0) return (int)c;
+  return (int)s;
+}
+
 }  // namespace ffnk

@@ -41,11 +41,15 @@ def test_workspace_bytes():
 def test_tile_table_entries():
     big = _lib.tile_config(_lib.OP_FFN_UP, 32768, 4096, 14336)
     assert big["path"] == _lib.PATH_MFMA_TILED and big["block_m"] == 256 and big["direct_lds"] == 1
-    assert big["block_k"] == 64 and big["lds_stages"] == 2
+    assert big["block_k"] == 32 and big["lds_stages"] == 4  # direct global->LDS ring
+    dec = _lib.tile_config(_lib.OP_FFN_FWD, 8, 4096, 14336)
+    assert dec["path"] == _lib.PATH_STREAM and dec["lds_stages"] == 0 and dec["block_m"] == 16
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 64, 4096, 14336)["split_k"] >= 4
+    assert _lib.tile_config(_lib.OP_FFN_FWD, 65, 4096, 14336)["path"] == _lib.PATH_MFMA_TILED
     small = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 1024, 1024)
     assert small["block_m"] * small["block_n"] < 256 * 256  # small problems get small tiles
     tail = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 72, 1024)
-    assert tail["direct_lds"] == 0
+    assert tail["direct_lds"] == 0 and tail["block_k"] == 64 and tail["lds_stages"] == 2
     dw = _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)
     assert dw["split_k"] > 1
     with pytest.raises(ValueError):

@@ -195,6 +195,43 @@ def test_ffn_fwd_vs_oracle(dev, M, d, h, p):
     assert_close_bf16_pair(out, om.ffn_blend(w.x, w.W, w.mask), "vs blend-form bf16 module")
 
 
+# decode shapes (M <= 64, d and h multiples of 256): the weight-streaming kernels
+DECODE_SHAPES = [(1, "visual"), (1, "text"), (2, "bernoulli"), (8, "bernoulli"), (15, "bernoulli"), (16, "visual"),
+                 (17, "bernoulli"), (32, "bernoulli"), (33, "text"), (47, "bernoulli"), (64, "bernoulli"),
+                 (64, "visual")]
+
+
+@pytest.mark.parametrize("M,kind", DECODE_SHAPES)
+@pytest.mark.parametrize("d,h", [(256, 512), (512, 1792)])
+def test_ffn_decode_path_vs_oracle(dev, M, kind, d, h):
+    note(f"ffn decode M={M} kind={kind} d={d} h={h}")
+    assert _lib.tile_config(_lib.OP_FFN_FWD, M, d, h)["path"] == _lib.PATH_STREAM
+    w = wl.cfg5_ffn_decode(M, kind, seed=M, d=d, h=h)
+    w = wl.FFNWorkload(w.name, w.x, {k: (v.float() * 2.5).to(torch.bfloat16) for k, v in w.W.items()}, w.mask)
+    out = MaskedFFN.apply(*w.to(dev).op_args())
+    torch.cuda.synchronize()
+    assert_close(out, cref.ffn_fwd(w.x, w.W, w.mask, round_mid=True), f"decode {M} {kind}")
+    # an absent modality's weights are never read: poison them
+    if kind in ("visual", "text"):
+        W = dict(w.W)
+        for k in (("u1", "u2", "u3") if kind == "visual" else ("w1", "w2", "w3")):
+            W[k] = torch.full_like(W[k], float("nan"))
+        out2 = MaskedFFN.apply(*wl.FFNWorkload("p", w.x, W, w.mask).to(dev).op_args())
+        assert torch.equal(out2, out)
+
+
+def test_ffn_decode_matches_tiled_path_rows(dev):
+    """The same rows run as a decode call and inside a larger (tiled-path) call agree to bf16 accuracy."""
+    note("ffn decode vs tiled")
+    d, h = 512, 1024
+    big = wl.make_ffn("t", 200, d, h, torch.rand(200, generator=torch.Generator().manual_seed(3)) < 0.5, seed=4,
+                      w_std=0.05).to(dev)
+    full = MaskedFFN.apply(*big.op_args())
+    small = wl.FFNWorkload("s", big.x[:48].contiguous(), big.W, big.mask[:48].contiguous())
+    part = MaskedFFN.apply(*small.op_args())
+    assert_close_bf16_pair(part, full[:48].float().cpu(), "decode rows vs tiled rows")
+
+
 def test_ffn_cfg2(dev):
     note("ffn cfg2")
     w = wl.cfg2_ffn_fwd()
