@@ -1,7 +1,7 @@
 """Headline benchmark: MaskedFFN forward, routed bf16 TFLOP/s at d=4096, h=14336, M=32768 on one
 MI355X (BASELINE.json's metric, `configs[3]`).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4|cfg2|decode64|...]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4|cfg2|decode1v|decode1t|decode8|decode32|decode64]
 
 A step is one MaskedFFN.apply over the whole synthetic batch (row partition + up-projection with
 SwiGLU + down-projection), inputs already resident in HBM.  Prints ONE JSON line.
@@ -53,7 +53,7 @@ class HipEvents:
             self.hip.hipEventDestroy(h)
 
 
-def _ffn_call_with_events(w, events):
+def _ffn_call_with_events(w, events, W=None):
     """One ffnk_masked_ffn_fwd_ev call (same path as MaskedFFN.apply) recording stage events."""
     import torch
     from ffn_kernel_amd import _lib
@@ -61,7 +61,7 @@ def _ffn_call_with_events(w, events):
     x = w.x
     M, d = x.shape
     h = w.h
-    W = w.W
+    W = W or w.W
     out = torch.empty((M, d), device=x.device, dtype=torch.bfloat16)
     ws = torch.empty(_lib.workspace_bytes(_lib.OP_FFN_FWD, M, d, h), dtype=torch.uint8, device=x.device)
     rc = lib.ffnk_masked_ffn_fwd_ev(x.data_ptr(), x.stride(0), W["w1"].data_ptr(), W["w3"].data_ptr(),
@@ -79,11 +79,17 @@ def _cpu_baseline(w, rows: int) -> dict:
     import torch
     from oracle import modules as om
     torch.set_num_threads(os.cpu_count() or 1)
-    x = w.x[:rows].cpu()
-    mask = w.mask[:rows].cpu()
     W = {k: v.cpu() for k, v in w.W.items()}
     with torch.no_grad():
-        om.ffn_blend(x[: max(rows // 8, 1)], W, mask[: max(rows // 8, 1)])  # warm-up
+        probe = min(256, rows)
+        om.ffn_blend(w.x[:probe].cpu(), W, w.mask[:probe].cpu())  # warm-up
+        t0 = time.perf_counter()
+        om.ffn_blend(w.x[:probe].cpu(), W, w.mask[:probe].cpu())
+        per_row = (time.perf_counter() - t0) / probe
+        # about 5 s per timed run, three runs
+        rows = max(probe, min(rows, int(5.0 / max(per_row, 1e-9))))
+        x = w.x[:rows].cpu()
+        mask = w.mask[:rows].cpu()
         times = []
         for _ in range(3):
             t0 = time.perf_counter()
@@ -104,7 +110,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg4")
-    ap.add_argument("--cpu-rows", type=int, default=512, help="rows of the workload timed on the CPU (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=1 << 30,
+                    help="upper bound on the rows of the workload timed on the CPU (0 = skip); the sample is "
+                         "sized to about 5 s per run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (rows are independent, so more GPUs "
@@ -118,32 +126,56 @@ def main() -> int:
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "copy1g":
+        # Calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of exactly 1 GiB
+        # (reads 1 GiB, writes 1 GiB per launch).  Not a benchmark of this library.
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": "copy1g", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
+        return 0
     if args.workload == "cfg4":
         w_cpu = wl.cfg4_ffn_fwd()
     elif args.workload == "cfg2":
         w_cpu = wl.cfg2_ffn_fwd()
     elif args.workload.startswith("decode"):
-        w_cpu = wl.cfg5_ffn_decode(int(args.workload[6:] or 64))
+        spec = args.workload[6:] or "64"
+        kind = {"v": "visual", "t": "text"}.get(spec[-1], "bernoulli")
+        w_cpu = wl.cfg5_ffn_decode(int(spec.rstrip("vt")), kind)
     else:
         raise SystemExit(f"unknown workload {args.workload}")
     w = w_cpu.to(dev)
-    op_args = w.op_args()
     M = w.x.shape[0]
+    tile = _lib.tile_config(_lib.OP_FFN_UP, M, w.d, w.h)
+    decode = tile["path"] == _lib.PATH_STREAM
 
-    for _ in range(args.warmup):
-        MaskedFFN.apply(*op_args)
+    # Decode calls are bound by streaming the weights: rotate three distinct weight sets (each larger
+    # than the 256 MB Infinity Cache) so that what is measured is HBM, not cache.
+    weight_sets = [w.W]
+    if decode:
+        for r in (1, 2):
+            g = torch.Generator().manual_seed(9000 + r)
+            weight_sets.append({k: (torch.randn(v.shape, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+                                for k, v in w_cpu.W.items()})
+    arg_sets = [wl.FFNWorkload(w.name, w.x, W, w.mask).op_args() for W in weight_sets]
+    ns = len(arg_sets)
+
+    for i in range(args.warmup):
+        MaskedFFN.apply(*arg_sets[i % ns])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        MaskedFFN.apply(*op_args)
+    for i in range(args.steps):
+        MaskedFFN.apply(*arg_sets[i % ns])
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # Dominant kernel, timed with HIP events on the launch stream inside the same C-ABI call.
+    # Stage durations from HIP events recorded on the launch stream inside the same C-ABI call.
     ev = HipEvents(3)
     up_ms, down_ms = [], []
-    for _ in range(max(args.steps, 3)):
-        _ffn_call_with_events(w, ev)
+    for i in range(max(args.steps, 3)):
+        _ffn_call_with_events(w, ev, weight_sets[i % ns])
         torch.cuda.synchronize()
         up_ms.append(ev.elapsed_ms(0, 1))
         down_ms.append(ev.elapsed_ms(1, 2))
@@ -151,13 +183,19 @@ def main() -> int:
     up_avg = sum(up_ms) / len(up_ms)
     down_avg = sum(down_ms) / len(down_ms)
 
-    tile = _lib.tile_config(_lib.OP_FFN_UP, M, w.d, w.h)
-    decode = tile["path"] == _lib.PATH_STREAM or M <= 64
     if decode:
-        # weight-streaming regime: algorithmic bytes of the whole call over its duration
-        achieved = w_cpu.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9
+        # weight-streaming regime: the dominant kernel is the up-projection stream (two of the three
+        # weight matrices of each modality present); its algorithmic bytes over its event-timed duration
+        nv = int(w_cpu.mask.sum())
+        present = int(nv > 0) + int(nv < M)
+        up_bytes = 2 * w.d * w.h * 2 * present + M * w.d * 2 + M
+        achieved = up_bytes / (up_avg * 1e-3) / 1e9
+        call_gbs = w_cpu.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": achieved / PEAK_HBM_GBS, "traffic": None, "kernel": "whole call (up + down)"}
+                    "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                    "kernel": "stream_kernel (up-projection + SwiGLU)", "kernel_ms": up_avg,
+                    "down_and_reduce_ms": down_avg, "whole_call_GBps": call_gbs,
+                    "whole_call_frac": call_gbs / PEAK_HBM_GBS, "whole_call_bytes": w_cpu.algorithmic_bytes()}
     else:
         up_flops = 2 * M * w.d * w.h * 2  # gate and up projections of the routed branch
         achieved = up_flops / (up_avg * 1e-3) / 1e12

@@ -1,0 +1,69 @@
+"""Committed golden vectors (tests/golden/*.npz): the torch oracle must reproduce them on the CPU,
+and the HIP path must match them on the GPU."""
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import modules as om
+
+GOLD = Path(__file__).resolve().parent / "golden"
+
+
+def bf16(a: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def load(name):
+    return np.load(GOLD / name, allow_pickle=False)
+
+
+def test_oracle_reproduces_linear_golden():
+    g = load("linear_M37_K48_N40.npz")
+    x, Wv, Wt, grad = bf16(g["x"]), bf16(g["Wv"]), bf16(g["Wt"]), bf16(g["grad"])
+    mask = torch.from_numpy(g["mask"])
+    assert torch.allclose(om.linear_select(x, Wv, Wt, mask, torch.float64), torch.from_numpy(g["y"]), atol=1e-11, rtol=0)
+    dx, dWv, dWt = om.linear_backward_select(grad, x, Wv, Wt, mask, torch.float64)
+    for got, key in ((dx, "dx"), (dWv, "dWv"), (dWt, "dWt")):
+        assert torch.allclose(got, torch.from_numpy(g[key]), atol=1e-10, rtol=0)
+    perm, counts = om.stable_partition(g["mask"])
+    assert np.array_equal(perm, g["perm"]) and np.array_equal(counts, g["counts"])
+    # the reference's bf16 module form lands within bf16 accuracy of the golden values
+    assert om.error_report(om.linear_blend(x, Wv, Wt, mask), torch.from_numpy(g["y"]))["rel_l2"] < 1e-2
+
+
+def test_oracle_reproduces_ffn_golden():
+    for name in ("ffn_M19_d32_h48.npz", "ffn_decode_M5_d128_h128.npz"):
+        g = load(name)
+        W = {k: bf16(g[k]) for k in ("w1", "w2", "w3", "u1", "u2", "u3")}
+        x, mask = bf16(g["x"]), torch.from_numpy(g["mask"])
+        got = om.ffn_select(x, W, mask, torch.float64, round_intermediate=True)
+        assert torch.allclose(got, torch.from_numpy(g["out_round_mid"]), atol=1e-9, rtol=0)
+        if "out" in g.files:
+            assert torch.allclose(om.ffn_select(x, W, mask, torch.float64), torch.from_numpy(g["out"]), atol=1e-10, rtol=0)
+
+
+@pytest.mark.gpu
+def test_hip_path_matches_golden(dev):
+    from ffn_kernel_amd import MaskedFFN, MaskedLinear
+    from helpers import assert_close, note
+    note("golden linear")
+    g = load("linear_M37_K48_N40.npz")
+    x = bf16(g["x"]).to(dev).requires_grad_(True)
+    Wv = bf16(g["Wv"]).to(dev).requires_grad_(True)
+    Wt = bf16(g["Wt"]).to(dev).requires_grad_(True)
+    mask = torch.from_numpy(g["mask"]).to(dev)
+    y = MaskedLinear.apply(x, Wv.T, Wt.T, mask)
+    y.backward(bf16(g["grad"]).to(dev))
+    assert_close(y, torch.from_numpy(g["y"]), "golden y")
+    assert_close(x.grad, torch.from_numpy(g["dx"]), "golden dx")
+    assert_close(Wv.grad, torch.from_numpy(g["dWv"]), "golden dWv")
+    assert_close(Wt.grad, torch.from_numpy(g["dWt"]), "golden dWt")
+    for name in ("ffn_M19_d32_h48.npz", "ffn_decode_M5_d128_h128.npz"):
+        note("golden " + name)
+        g = load(name)
+        W = {k: bf16(g[k]).to(dev) for k in ("w1", "w2", "w3", "u1", "u2", "u3")}
+        out = MaskedFFN.apply(bf16(g["x"]).to(dev), W["w1"].T, W["w2"].T, W["w3"].T, W["u1"].T, W["u2"].T, W["u3"].T,
+                              torch.from_numpy(g["mask"]).to(dev))
+        assert_close(out, torch.from_numpy(g["out_round_mid"]), "golden ffn")
