@@ -3,6 +3,7 @@
 Drop-in for the `ffn_kernel` package of wenhaoli-xmu/ffn_kernel (ffn_kernel/__init__.py:1):
     from ffn_kernel_amd import MaskedLinear, MaskedFFN
 """
+from .modules import MaskedFFNModule, MaskedLinearModule
 from .ops import MaskedFFN, MaskedLinear, masked_ffn_forward, masked_linear_backward, masked_linear_forward
 
-__all__ = ["MaskedLinear", "MaskedFFN", "masked_linear_forward", "masked_linear_backward", "masked_ffn_forward"]
+__all__ = ["MaskedLinear", "MaskedFFN", "MaskedLinearModule", "MaskedFFNModule", "masked_linear_forward", "masked_linear_backward", "masked_ffn_forward"]

@@ -334,3 +334,39 @@ def test_linear_bwd_cfg3(dev):
     tot = (w.grad.double().T @ w.x.double())
     gv, gt = dbv.T.double().cpu(), dbt.T.double().cpu()
     assert ((gv + gt - tot).abs() <= 2.0 ** -8 * (gv.abs() + gt.abs()) + 1e-6).all()
+
+
+# ------------------------------------------------------------------ nn.Module wrappers (3-D inputs)
+def test_modules_match_reference_modules(dev):
+    """The wrappers load the reference PyTorch modules' state_dicts and reproduce them on [B, S, D]
+    inputs, forward (both) and backward (linear), as test_linear.py:92-102 compares them."""
+    note("module wrappers")
+    from ffn_kernel_amd import MaskedFFNModule, MaskedLinearModule
+    torch.manual_seed(0)
+    B, S, D, Hh = 2, 150, 64, 128
+    x = torch.randn(B, S, D).to(torch.bfloat16)
+    mask = torch.rand(B, S) < 0.4
+    ref_lin = om.TorchLinear(D, 96).bfloat16()
+    mod = MaskedLinearModule(D, 96, device=dev)
+    mod.load_state_dict(ref_lin.state_dict())
+    xd = x.to(dev).requires_grad_(True)
+    y = mod(xd, mask.to(dev))
+    assert y.shape == (B, S, 96)
+    y.sum().backward()
+    xr = x.float().requires_grad_(True)
+    ref = om.TorchLinear(D, 96)
+    ref.load_state_dict({k: v.float() for k, v in ref_lin.state_dict().items()})
+    yr = ref(xr, mask)
+    yr.sum().backward()
+    assert_close(y, yr.detach().double(), "module y")
+    assert_close(xd.grad, xr.grad.double(), "module dx")
+    assert_close(mod.linear_v.weight.grad, ref.linear_v.weight.grad.double(), "module dWv")
+    assert_close(mod.linear_t.weight.grad, ref.linear_t.weight.grad.double(), "module dWt")
+    ref_ffn = om.TorchFFN(D, Hh).bfloat16()
+    ffn = MaskedFFNModule(D, Hh, device=dev)
+    ffn.load_state_dict(ref_ffn.state_dict())
+    out = ffn(x.to(dev), mask.to(dev))
+    assert out.shape == (B, S, D)
+    assert_close_bf16_pair(out, ref_ffn(x, mask).float(), "module ffn vs reference module")
+    out2 = ffn(x.to(dev).flatten(0, 1), mask.to(dev).flatten())
+    assert torch.equal(out2, out.flatten(0, 1))
