@@ -99,6 +99,10 @@ bool direct_ok(int64_t K, int64_t gathered_rows, int64_t lda, int64_t ldb) {
 
 bool use_stream_path(int64_t M, int64_t d, int64_t h) { return stream_shape_ok(M, d, h); }
 
+int down_splits(int64_t M, int64_t d, int64_t h) {
+  return stream_down_splits(d, h, stream_rows_per_block((int)M, false), stream_waves_per_block((int)M, false));
+}
+
 }  // namespace
 
 extern "C" {
@@ -123,7 +127,7 @@ size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
       // perm + counts + the [M, h] bf16 intermediate in routed order (N = h); the streaming path
       // adds the fp32 split-K partials of the down projection.
       return route_ws_bytes(M) + ws_align((size_t)M * round_up64(N, 8) * 2) +
-             (use_stream_path(M, K, N) ? ws_align((size_t)stream_down_splits(K, N) * M * K * 4) : 0);
+             (use_stream_path(M, K, N) ? ws_align((size_t)down_splits(M, K, N) * M * K * 4) : 0);
     case FFNK_OP_LINEAR_BWD: {
       const BwdPlan a = plan_bwd(M, K, N, true), b = plan_bwd(M, K, N, false);
       return a.total > b.total ? a.total : b.total;
@@ -179,7 +183,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
     out->waves_n = 1;
     out->lds_stages = 0;
     out->group_m = 1;
-    out->split_k = 4 * (up ? 1 : stream_down_splits(K, N));
+    out->split_k = stream_waves_per_block((int)M, up) * (up ? 1 : down_splits(M, K, N));
     out->direct_lds = 0;
   }
   return FFNK_OK;
@@ -285,20 +289,22 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
 
   if (use_stream_path(M, d, h)) {
     float* P = reinterpret_cast<float*>(wsb + r.bytes + ws_align((size_t)M * ldh * 2));
-    const int splits = stream_down_splits(d, h);
+    const int splits = down_splits(M, d, h);
     FFNK_HIP(mark(0), "event record");
     StreamArgs u;
     u.X = x; u.ldx = x_stride_m; u.gather_x = 1; u.mask = mask; u.M = (int)M;
     u.W0[0] = W1; u.W0[1] = U1; u.W1[0] = W3; u.W1[1] = U3; u.ldw = up_stride_n;
-    u.Nrows = (int)h; u.K = (int)d; u.splits = 1; u.H = H; u.ldh = ldh; u.P = nullptr;
+    u.Nrows = (int)h; u.K = (int)d; u.splits = 1; u.H = H; u.ldh = ldh; u.P = nullptr; u.out = nullptr; u.ldo = 0;
     FFNK_HIP(launch_stream_up(u, stream), "streaming up-projection");
     FFNK_HIP(mark(1), "event record");
     StreamArgs dn;
     dn.X = H; dn.ldx = ldh; dn.gather_x = 0; dn.mask = mask; dn.M = (int)M;
     dn.W0[0] = W2; dn.W0[1] = U2; dn.W1[0] = dn.W1[1] = nullptr; dn.ldw = down_stride_n;
-    dn.Nrows = (int)d; dn.K = (int)h; dn.splits = splits; dn.H = nullptr; dn.ldh = 0; dn.P = P;
+    dn.Nrows = (int)d; dn.K = (int)h; dn.splits = splits; dn.H = nullptr; dn.ldh = 0;
+    dn.P = splits > 1 ? P : nullptr; dn.out = out; dn.ldo = out_stride_m;
     FFNK_HIP(launch_stream_down(dn, stream), "streaming down-projection");
-    FFNK_HIP(launch_stream_reduce(P, splits, (int)M, (int)d, mask, out, out_stride_m, stream), "streaming reduce");
+    if (splits > 1)
+      FFNK_HIP(launch_stream_reduce(P, splits, (int)M, (int)d, mask, out, out_stride_m, stream), "streaming reduce");
     FFNK_HIP(mark(2), "event record");
     return FFNK_OK;
   }

@@ -56,11 +56,13 @@ struct StreamArgs {
   int64_t ldw;
   int Nrows, K, splits;            // K % 256 == 0; splits > 1 only for the down projection
   uint16_t* H; int64_t ldh;        // up-projection output, routed order [M, Nrows]
-  float* P;                        // down-projection partials [splits][M][Nrows] (routed order)
+  float* P;                        // down-projection partials [splits][M][Nrows] (routed order), or NULL:
+  uint16_t* out; int64_t ldo;      // ... splits == 1 and the result goes straight to out (token order)
 };
 // Shape of the streaming kernels for M rows (reported through ffnk_tile_config).
 int stream_rows_per_block(int M, bool dual);  // weight rows (of each matrix) per workgroup
 int stream_chunk_k(int M, bool dual);         // K elements per streamed chunk
+int stream_waves_per_block(int M, bool dual); // wavefronts sharing one workgroup's K range
 hipError_t launch_stream_up(const StreamArgs& a, hipStream_t stream);
 hipError_t launch_stream_down(const StreamArgs& a, hipStream_t stream);
 // out[token row of p, n] = bf16(sum_s P[s][p][n])

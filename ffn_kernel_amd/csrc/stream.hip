@@ -17,16 +17,6 @@
 namespace ffnk {
 
 constexpr int kSK = 128;                    // K elements per streamed chunk
-constexpr int kSWaves = 4;                  // wavefronts per workgroup
-constexpr int kSThreads = kSWaves * kWave;
-#ifndef FFNK_RT_UP1
-#define FFNK_RT_UP1 1
-#endif
-#ifndef FFNK_RT_DOWN1
-#define FFNK_RT_DOWN1 1
-#endif
-constexpr int kRtUp1 = FFNK_RT_UP1;      // row tiles per wavefront for M <= 16, up-projection
-constexpr int kRtDown1 = FFNK_RT_DOWN1;  // ... and down-projection
 constexpr int kSMaxM = 64;
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -61,7 +51,7 @@ struct StreamTile {
 // token-row fragments are both loaded straight from global memory into MFMA operand registers
 // (the token rows are few and L1/L2-resident), one 128-element K chunk ahead of the MFMAs.
 // acc = W_frag (16 rows x 32 k) * X_frag (32 k x 16 token rows) per 16x16 tile.
-template <int NTM, bool DUAL, int RT, int KS>
+template <int NTM, bool DUAL, int RT, int KS, int NWV>
 __device__ __forceinline__ void stream_rows(const StreamArgs& a, const StreamTile& t, const int* s_perm,
                                             float* s_red) {
   constexpr int CK = KS * 32;  // K elements per chunk (t.c0 / t.nc count chunks of this size)
@@ -128,7 +118,7 @@ __device__ __forceinline__ void stream_rows(const StreamArgs& a, const StreamTil
     }
   }
 
-  // The four wavefronts of the workgroup hold partial sums over their quarters of the K range:
+  // The wavefronts of the workgroup hold partial sums over their shares of the K range:
   // add them up through LDS (fixed order: deterministic), wave 0 finishes.
   const int wave = threadIdx.x >> 6;
   if (wave > 0) {
@@ -141,7 +131,7 @@ __device__ __forceinline__ void stream_rows(const StreamArgs& a, const StreamTil
   __syncthreads();
   if (wave > 0) return;
 #pragma unroll
-  for (int v = 0; v < kSWaves - 1; ++v)
+  for (int v = 0; v < NWV - 1; ++v)
 #pragma unroll
     for (int w = 0; w < NW; ++w)
 #pragma unroll
@@ -163,10 +153,19 @@ __device__ __forceinline__ void stream_rows(const StreamArgs& a, const StreamTil
           v2.x = pack2bf(swiglu(g[0], u[0]), swiglu(g[1], u[1]));
           v2.y = pack2bf(swiglu(g[2], u[2]), swiglu(g[3], u[3]));
           *reinterpret_cast<uint2*>(a.H + (int64_t)(t.p0 + row) * a.ldh + n_out) = v2;
-        } else {
+        } else if (a.P != nullptr) {
           const f32x4_t o = acc[r][m];
           *reinterpret_cast<float4*>(a.P + ((int64_t)t.split * a.M + (t.p0 + row)) * a.Nrows + n_out) =
               make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+          // single split: this workgroup holds the complete sums, store the output row directly
+          const f32x4_t o = acc[r][m];
+          uint2 v2;
+          v2.x = pack2bf(o[0], o[1]);
+          v2.y = pack2bf(o[2], o[3]);
+          uint16_t* dst = a.out + (int64_t)s_perm[t.p0 + row] * a.ldo + n_out;
+          if ((reinterpret_cast<uintptr_t>(dst) & 7) == 0) *reinterpret_cast<uint2*>(dst) = v2;
+          else { dst[0] = f2bf(o[0]); dst[1] = f2bf(o[1]); dst[2] = f2bf(o[2]); dst[3] = f2bf(o[3]); }
         }
       }
     }
@@ -176,17 +175,20 @@ __device__ __forceinline__ void stream_rows(const StreamArgs& a, const StreamTil
 // NTM_MAX = ceil(M / 16), known on the host: bounds the register budget so that small-M calls
 // run at higher occupancy.  A workgroup = 16 weight rows (of each matrix) x one K range; its four
 // wavefronts take a quarter of the range each.
-template <int NTM_MAX, bool DUAL, int RT, int KS, int OCC>
-__global__ __launch_bounds__(kSThreads, OCC) void stream_kernel(const StreamArgs a) {
+template <int NTM_MAX, bool DUAL, int RT, int KS, int NWV, int OCC>
+__global__ __launch_bounds__(NWV * kWave, OCC) void stream_kernel(const StreamArgs a) {
   __shared__ int s_perm[kSMaxM];
   __shared__ int s_nvis;
-  __shared__ __attribute__((aligned(16))) float s_red[(kSWaves - 1) * RT * (DUAL ? 2 : 1) * NTM_MAX * 64 * 4];
+  __shared__ __attribute__((aligned(16))) float s_red[(NWV - 1) * RT * (DUAL ? 2 : 1) * NTM_MAX * 64 * 4];
   const int n_vis = route_small(a.mask, a.M, s_perm, &s_nvis);
 
   // blockIdx -> (group, split, row block)
   const int row_blocks = cdiv(a.Nrows, 16 * RT);
-  const int per_grp = row_blocks * a.splits;
   StreamTile t;
+  // Group-major order: all workgroups of the visual group, then all of the text group.  (Interleaving
+  // the groups was measured 1.5x slower when one modality is absent: its empty workgroups still take
+  // their turn in the round-robin placement over CUs, so the real ones pile up on half of the CUs.)
+  const int per_grp = row_blocks * a.splits;
   t.grp = blockIdx.x / per_grp;
   const int rem = blockIdx.x % per_grp;
   t.split = rem / row_blocks;
@@ -200,16 +202,16 @@ __global__ __launch_bounds__(kSThreads, OCC) void stream_kernel(const StreamArgs
   const int n128 = a.K / kSK;
   const int cps = cdiv(n128, a.splits);
   const int b0 = min(t.split * cps, n128) * PER128, b1 = min((t.split + 1) * cps, n128) * PER128;
-  const int per_wave = cdiv(b1 - b0, kSWaves);
+  const int per_wave = cdiv(b1 - b0, NWV);
   const int wave = threadIdx.x >> 6;
   t.c0 = min(b0 + wave * per_wave, b1);
   t.nc = min(t.c0 + per_wave, b1) - t.c0;
 
   const int ntm = cdiv(t.mg, 16);  // uniform over the workgroup
-  if (NTM_MAX >= 4 && ntm >= 4) stream_rows<(NTM_MAX >= 4 ? 4 : 1), DUAL, RT, KS>(a, t, s_perm, s_red);
-  else if (NTM_MAX >= 3 && ntm == 3) stream_rows<(NTM_MAX >= 3 ? 3 : 1), DUAL, RT, KS>(a, t, s_perm, s_red);
-  else if (NTM_MAX >= 2 && ntm == 2) stream_rows<(NTM_MAX >= 2 ? 2 : 1), DUAL, RT, KS>(a, t, s_perm, s_red);
-  else stream_rows<1, DUAL, RT, KS>(a, t, s_perm, s_red);
+  if (NTM_MAX >= 4 && ntm >= 4) stream_rows<(NTM_MAX >= 4 ? 4 : 1), DUAL, RT, KS, NWV>(a, t, s_perm, s_red);
+  else if (NTM_MAX >= 3 && ntm == 3) stream_rows<(NTM_MAX >= 3 ? 3 : 1), DUAL, RT, KS, NWV>(a, t, s_perm, s_red);
+  else if (NTM_MAX >= 2 && ntm == 2) stream_rows<(NTM_MAX >= 2 ? 2 : 1), DUAL, RT, KS, NWV>(a, t, s_perm, s_red);
+  else stream_rows<1, DUAL, RT, KS, NWV>(a, t, s_perm, s_red);
 }
 
 // out[perm[p], n] = bf16(sum_s P[s][p][n]); one workgroup per (routed row, 1024 columns).
@@ -238,13 +240,25 @@ __global__ __launch_bounds__(256) void stream_reduce_kernel(const float* __restr
   }
 }
 
-// Row tiles per wavefront: two where registers allow, so that a token-row fragment is used twice.
-template <int NTM_MAX, bool DUAL>
-struct StreamShape {
-  static constexpr int RT = DUAL ? (NTM_MAX <= 1 ? kRtUp1 : 2) : (NTM_MAX <= 1 ? kRtDown1 : 2);
-  static constexpr int KS = (DUAL && NTM_MAX >= 2) ? 2 : 4;  // k-steps per chunk: 64 or 128 elements
-  static constexpr int OCC = DUAL ? (NTM_MAX == 1 ? (RT == 1 ? 4 : 2) : 2) : (NTM_MAX == 1 ? (RT == 1 ? 4 : 3) : 2);
+// Shape of the streaming kernel per (m-tiles, projection): RT row tiles of 16 weight rows per
+// wavefront (a token-row fragment is then used RT times), KS 32-element k-steps per chunk, NWV
+// wavefronts per workgroup sharing the K range, OCC waves per SIMD the register budget allows.
+#ifndef FFNK_S_UP1
+#define FFNK_S_UP1 1, 4, 4, 4
+#endif
+#ifndef FFNK_S_DOWN1
+#define FFNK_S_DOWN1 1, 4, 16, 4
+#endif
+template <int RT_, int KS_, int NWV_, int OCC_>
+struct StreamShapeV {
+  static constexpr int RT = RT_, KS = KS_, NWV = NWV_, OCC = OCC_;
 };
+template <int NTM_MAX, bool DUAL>
+struct StreamShape : StreamShapeV<2, (DUAL ? 2 : 4), 4, 2> {};
+template <>
+struct StreamShape<1, true> : StreamShapeV<FFNK_S_UP1> {};
+template <>
+struct StreamShape<1, false> : StreamShapeV<FFNK_S_DOWN1> {};
 
 int stream_rows_per_block(int M, bool dual) {
   switch (cdiv(M, 16)) {
@@ -252,6 +266,15 @@ int stream_rows_per_block(int M, bool dual) {
     case 2: return 16 * (dual ? StreamShape<2, true>::RT : StreamShape<2, false>::RT);
     case 3: return 16 * (dual ? StreamShape<3, true>::RT : StreamShape<3, false>::RT);
     default: return 16 * (dual ? StreamShape<4, true>::RT : StreamShape<4, false>::RT);
+  }
+}
+
+int stream_waves_per_block(int M, bool dual) {
+  switch (cdiv(M, 16)) {
+    case 1: return dual ? StreamShape<1, true>::NWV : StreamShape<1, false>::NWV;
+    case 2: return dual ? StreamShape<2, true>::NWV : StreamShape<2, false>::NWV;
+    case 3: return dual ? StreamShape<3, true>::NWV : StreamShape<3, false>::NWV;
+    default: return dual ? StreamShape<4, true>::NWV : StreamShape<4, false>::NWV;
   }
 }
 
@@ -268,12 +291,13 @@ template <int NTM_MAX, bool DUAL>
 static void launch_stream_n(const StreamArgs& a, hipStream_t stream) {
   using S = StreamShape<NTM_MAX, DUAL>;
   const int blocks = 2 * cdiv(a.Nrows, 16 * S::RT) * a.splits;
-  hipLaunchKernelGGL((stream_kernel<NTM_MAX, DUAL, S::RT, S::KS, S::OCC>), dim3(blocks), dim3(kSThreads), 0, stream, a);
+  hipLaunchKernelGGL((stream_kernel<NTM_MAX, DUAL, S::RT, S::KS, S::NWV, S::OCC>), dim3(blocks), dim3(S::NWV * kWave), 0, stream, a);
 }
 
 template <bool DUAL>
 static hipError_t launch_stream(const StreamArgs& a, hipStream_t stream) {
   if (a.M < 1 || a.M > kSMaxM || a.K % kSK != 0 || a.splits < 1) return hipErrorInvalidValue;
+  if (!DUAL && a.P == nullptr && (a.splits != 1 || a.out == nullptr)) return hipErrorInvalidValue;
   switch (cdiv(a.M, 16)) {
     case 1: launch_stream_n<1, DUAL>(a, stream); break;
     case 2: launch_stream_n<2, DUAL>(a, stream); break;

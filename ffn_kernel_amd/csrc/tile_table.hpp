@@ -51,19 +51,20 @@ inline bool stream_shape_ok(int64_t M, int64_t d, int64_t h) {
   return M >= 1 && M <= kStreamMaxM && d >= 128 && h >= 128 && d % 128 == 0 && h % 128 == 0 && d % 16 == 0;
 }
 
-// Split-K factor of the streamed down-projection.  A workgroup covers 16 weight rows x one K
-// range (its four wavefronts take a quarter each); aim at about 16 wavefronts per CU and per
-// modality, keep at least four 128-element chunks per workgroup, and prefer a split that gives
-// every wavefront the same number of chunks.
-inline int stream_down_splits(int64_t d, int64_t h) {
-  const int64_t row_blocks = cdiv64(d, 16);
+// Split-K factor of the streamed down-projection.  A workgroup covers `rows_per_block` weight rows
+// x one K range that its `waves` wavefronts share.  Aim at about 16 wavefronts per CU and per
+// modality, keep at least four 128-element chunks per wavefront, prefer a split that gives every
+// wavefront the same number of chunks.  1 means no cross-workgroup split: the kernel then stores
+// the output itself and no reduce pass runs.
+inline int stream_down_splits(int64_t d, int64_t h, int rows_per_block, int waves) {
+  const int64_t row_blocks = cdiv64(d, rows_per_block);
   const int64_t chunks = h / 128;
-  int64_t s = cdiv64(4 * kCus, row_blocks);
-  if (s > chunks / 4) s = chunks / 4;
+  int64_t s = cdiv64((int64_t)16 * kCus, row_blocks * waves);
+  if (s > chunks / (4 * waves)) s = chunks / (4 * waves);
   if (s > 16) s = 16;
   if (s < 1) s = 1;
   for (int64_t c = s; c >= 1 && c * 2 > s; --c)
-    if (chunks % (c * 4) == 0) return (int)c;
+    if (chunks % (c * waves) == 0) return (int)c;
   return (int)s;
 }
 
