@@ -389,8 +389,8 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]
   uint16_t* XT = reinterpret_cast<uint16_t*>(wsb + p.off_xt);  // [K, ldt]
   float* P = reinterpret_cast<float*>(wsb + p.off_p);
-  FFNK_HIP(launch_gather_transpose(g, g_stride_m, r.perm, r.counts, GT, p.ldt, (int)M, (int)N, stream), "g transpose");
-  FFNK_HIP(launch_gather_transpose(x, x_stride_m, r.perm, r.counts, XT, p.ldt, (int)M, (int)K, stream), "x transpose");
+  FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)N, GT, x, x_stride_m, (int)K, XT, p.ldt, r.perm, r.counts,
+                                    (int)M, stream), "g / x transpose");
   SplitKArgs s;
   s.A = p.dw_k_contig ? GT : XT; s.lda = p.ldt;
   s.B = p.dw_k_contig ? XT : GT; s.ldb = p.ldt;

@@ -223,19 +223,19 @@ __device__ __forceinline__ void gemm_mainloop_ring(const RingLanes<Cfg>& rl,
     mfmas(1);
     if (full) {
       // Issue order inside the (branch-free) steady-state iteration: one LDS read after each of
-      // the first TM+TN MFMAs of a K step, one global->LDS load after each of the next ones.
+      // the first TM+TN MFMAs of a K step; the L global->LDS loads spread evenly over the MFMAs
+      // that follow in the two K steps (a load takes about two MFMA slots to issue).
+      constexpr int FREE = NM - ND;                     // MFMAs per K step without an LDS read
+      constexpr int GAP = (2 * FREE) / L > 0 ? (2 * FREE) / L : 1;
 #pragma unroll
-      for (int q = 0; q < NM; ++q) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (q < ND) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        else if (q - ND < L) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      }
+      for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-      for (int q = 0; q < NM; ++q) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (q < ND) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        else if (q - ND + (NM - ND) < L) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      }
+        for (int q = 0; q < NM; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (q < ND) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          else if ((ks * FREE + (q - ND)) % GAP == 0 && (ks * FREE + (q - ND)) / GAP < L)
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
     }
   };
   int i0 = 0;

@@ -37,11 +37,12 @@ hipError_t launch_splitk_gemm(int tile, const SplitKArgs& g, hipStream_t stream)
 // dst[r, c] (row-major, ld_dst) = src[r * sr + c * sc] for r < rows, c < cols.
 hipError_t launch_strided_copy2d(const uint16_t* src, int64_t sr, int64_t sc, uint16_t* dst, int64_t ld_dst,
                                  int rows, int cols, hipStream_t stream);
-// dst[c, pos(p)] = src[perm[p], c]; routed columns padded per group to a multiple of 64 with
-// zeros: pos(p) = p for visual p, pad64(n_vis) + (p - n_vis) for text p.  dst is [cols, ld_dst].
-hipError_t launch_gather_transpose(const uint16_t* src, int64_t ld_src, const int32_t* perm,
-                                   const int32_t* counts, uint16_t* dst, int64_t ld_dst, int M, int cols,
-                                   hipStream_t stream);
+// For both (src, dst) pairs: dst[c, pos(p)] = src[perm[p], c]; routed columns padded per group to a
+// multiple of 64 with zeros: pos(p) = p for visual p, pad64(n_vis) + (p - n_vis) for text p.  dst is
+// [cols, ld_dst]; cols % 8 == 0 and 16-byte aligned source rows are required.
+hipError_t launch_gather_transpose2(const uint16_t* src0, int64_t ld0, int cols0, uint16_t* dst0,
+                                    const uint16_t* src1, int64_t ld1, int cols1, uint16_t* dst1, int64_t ld_dst,
+                                    const int32_t* perm, const int32_t* counts, int M, hipStream_t stream);
 // out_g[r * sr + c * sc] = bf16(sum_s P[g][s][r][c]) for g in {0, 1}.
 hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint16_t* out0, uint16_t* out1,
                                 int64_t sr, int64_t sc, hipStream_t stream);

@@ -40,45 +40,78 @@ hipError_t launch_strided_copy2d(const uint16_t* src, int64_t sr, int64_t sc, ui
 
 // dst[c, pos] = src[perm[p], c] over padded routed positions pos in [0, pad64(nv) + pad64(nt));
 // padding positions are written as zero so that they add nothing to a contraction over pos.
-__global__ __launch_bounds__(256) void gather_transpose_kernel(const uint16_t* __restrict__ src, int64_t ld_src,
-                                                               const int32_t* __restrict__ perm,
-                                                               const int32_t* __restrict__ counts,
-                                                               uint16_t* __restrict__ dst, int64_t ld_dst, int M,
-                                                               int cols) {
-  __shared__ uint16_t tile[kTt][kTt + 2];  // [routed position][column]
-  const int n_vis = counts[0];
-  const int vpad = (n_vis + 63) & ~63;
-  const int tpad = (M - n_vis + 63) & ~63;
-  const int pos0 = blockIdx.x * kTt;
-  if (pos0 >= vpad + tpad) return;  // grid is sized for the worst-case padding
+// blockIdx.z selects one of two (src, dst) pairs so that g and x are transposed in one launch.
+// 64 positions x 64 columns per block: 16-byte row reads, scalar transposing LDS writes, 16-byte
+// reads of the transposed tile, 16-byte stores (8 consecutive positions of one column).
+struct GatherTransposeArgs {
+  const uint16_t* src[2]; int64_t ld_src[2];
+  uint16_t* dst[2]; int64_t ld_dst;
+  int cols[2];
+  const int32_t* perm; const int32_t* counts;
+  int M;
+};
+
+__global__ __launch_bounds__(256) void gather_transpose_kernel(const GatherTransposeArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t tile[kTt][kTt + 8];  // [column][position]
+  const int z = blockIdx.z;
+  const int cols = a.cols[z];
   const int c0 = blockIdx.y * kTt;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  if (c0 >= cols) return;  // grid.y is sized for the wider of the two operands
+  const int n_vis = a.counts[0];
+  const int vpad = (n_vis + 63) & ~63;
+  const int tpad = (a.M - n_vis + 63) & ~63;
+  const int pos0 = blockIdx.x * kTt;
+  if (pos0 >= vpad + tpad) return;  // grid.x is sized for the worst-case padding
   // A 64-position block lies entirely inside one group because vpad is a multiple of 64.
   const bool text = pos0 >= vpad;
-  for (int i = ty; i < kTt; i += 4) {
+  const uint16_t* src = a.src[z];
+  const int64_t ld_src = a.ld_src[z];
+  const int t = threadIdx.x;
+  const int ch = t & 7;  // 8-column chunk of the 64-column tile
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int i = (t >> 3) + pass * 32;  // position inside the tile
     const int pos = pos0 + i;
     const int p = text ? n_vis + (pos - vpad) : pos;
-    const bool valid = text ? p < M : p < n_vis;
-    uint16_t v = 0;
-    const int c = c0 + tx;
-    if (valid && c < cols) v = src[(int64_t)perm[p] * ld_src + c];
-    tile[i][tx] = v;
+    const bool valid = text ? p < a.M : p < n_vis;
+    uint16_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int c = c0 + ch * 8;
+    if (valid) {
+      const uint16_t* row = src + (int64_t)a.perm[p] * ld_src;
+      if (c + 8 <= cols) {
+        *reinterpret_cast<uint4*>(v) = *reinterpret_cast<const uint4*>(row + c);  // cols % 8 == 0, 16-byte aligned rows
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (c + e < cols) v[e] = row[c + e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) tile[ch * 8 + e][i] = v[e];
   }
   __syncthreads();
-  for (int i = ty; i < kTt; i += 4) {
-    const int c = c0 + i;
-    if (c < cols) dst[(int64_t)c * ld_dst + pos0 + tx] = tile[tx][i];
+  uint16_t* dst = a.dst[z];
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int cc = (t >> 3) + pass * 32;  // column inside the tile
+    if (c0 + cc < cols)
+      *reinterpret_cast<uint4*>(dst + (int64_t)(c0 + cc) * a.ld_dst + pos0 + ch * 8) =
+          *reinterpret_cast<const uint4*>(&tile[cc][ch * 8]);
   }
 }
 
-hipError_t launch_gather_transpose(const uint16_t* src, int64_t ld_src, const int32_t* perm,
-                                   const int32_t* counts, uint16_t* dst, int64_t ld_dst, int M, int cols,
-                                   hipStream_t stream) {
-  if (M <= 0 || cols <= 0) return hipSuccess;
+hipError_t launch_gather_transpose2(const uint16_t* src0, int64_t ld0, int cols0, uint16_t* dst0,
+                                    const uint16_t* src1, int64_t ld1, int cols1, uint16_t* dst1, int64_t ld_dst,
+                                    const int32_t* perm, const int32_t* counts, int M, hipStream_t stream) {
+  if (M <= 0 || (cols0 <= 0 && cols1 <= 0)) return hipSuccess;
+  GatherTransposeArgs a;
+  a.src[0] = src0; a.ld_src[0] = ld0; a.dst[0] = dst0; a.cols[0] = cols0;
+  a.src[1] = src1; a.ld_src[1] = ld1; a.dst[1] = dst1; a.cols[1] = cols1;
+  a.ld_dst = ld_dst; a.perm = perm; a.counts = counts; a.M = M;
   const int max_pos = (int)round_up64(M, 64) + 64;  // >= pad64(nv) + pad64(nt) for every split of M
-  dim3 grid(cdiv(max_pos, kTt), cdiv(cols, kTt));
-  hipLaunchKernelGGL(gather_transpose_kernel, grid, dim3(256), 0, stream, src, ld_src, perm, counts, dst, ld_dst,
-                     M, cols);
+  const int max_cols = cols0 > cols1 ? cols0 : cols1;
+  dim3 grid(cdiv(max_pos, kTt), cdiv(max_cols, kTt), 2);
+  hipLaunchKernelGGL(gather_transpose_kernel, grid, dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 
