@@ -97,6 +97,12 @@ bool direct_ok(int64_t K, int64_t gathered_rows, int64_t lda, int64_t ldb) {
   return 256 * lda * 2 < k4g && 256 * ldb * 2 < k4g;
 }
 
+int g_force_tile = -1;  // tuner override, see ffnk_debug_force_tile
+
+int routed_tile(int64_t M, int64_t n_out, bool dual) {
+  return (g_force_tile >= 0 && g_force_tile < TILE_COUNT) ? g_force_tile : pick_routed_tile(M, n_out, dual);
+}
+
 bool use_stream_path(int64_t M, int64_t d, int64_t h) { return stream_shape_ok(M, d, h); }
 
 int down_splits(int64_t M, int64_t d, int64_t h) {
@@ -108,6 +114,12 @@ int down_splits(int64_t M, int64_t d, int64_t h) {
 extern "C" {
 
 int ffnk_version(void) { return FFNK_VERSION; }
+
+int ffnk_debug_force_tile(int tile) {
+  const int prev = g_force_tile;
+  g_force_tile = (tile >= 0 && tile < TILE_COUNT) ? tile : -1;
+  return prev;
+}
 
 const char* ffnk_last_error(void) { return g_err; }
 
@@ -223,7 +235,7 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
   g.C = y; g.ldc = y_stride_m;
   g.perm = r.perm; g.counts = r.counts;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
-  FFNK_HIP(launch_linear_gemm(pick_routed_tile(M, N, false), direct_ok(K, M, x_stride_m, w_stride_n), g, stream), "linear GEMM");
+  FFNK_HIP(launch_linear_gemm(routed_tile(M, N, false), direct_ok(K, M, x_stride_m, w_stride_n), g, stream), "linear GEMM");
   return FFNK_OK;
 }
 
@@ -317,7 +329,7 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
   up.C = H; up.ldc = ldh;
   up.perm = r.perm; up.counts = r.counts;
   up.M = (int)M; up.N = (int)h; up.K = (int)d;
-  FFNK_HIP(launch_up_gemm(pick_routed_tile(M, h, true), direct_ok(d, M, x_stride_m, up_stride_n), up, stream), "up-projection GEMM");
+  FFNK_HIP(launch_up_gemm(routed_tile(M, h, true), direct_ok(d, M, x_stride_m, up_stride_n), up, stream), "up-projection GEMM");
   FFNK_HIP(mark(1), "event record");
   GemmArgs dn;
   dn.A = H; dn.lda = ldh;
@@ -325,7 +337,7 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
   dn.C = out; dn.ldc = out_stride_m;
   dn.perm = r.perm; dn.counts = r.counts;
   dn.M = (int)M; dn.N = (int)d; dn.K = (int)h;
-  FFNK_HIP(launch_down_gemm(pick_routed_tile(M, d, false), direct_ok(h, 0, ldh, down_stride_n), dn, stream), "down-projection GEMM");
+  FFNK_HIP(launch_down_gemm(routed_tile(M, d, false), direct_ok(h, 0, ldh, down_stride_n), dn, stream), "down-projection GEMM");
   FFNK_HIP(mark(2), "event record");
   return FFNK_OK;
 }
@@ -383,7 +395,7 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   a.C = dx; a.ldc = dx_stride_m;
   a.perm = r.perm; a.counts = r.counts;
   a.M = (int)M; a.N = (int)K; a.K = (int)N;
-  FFNK_HIP(launch_linear_gemm(pick_routed_tile(M, K, false), direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
+  FFNK_HIP(launch_linear_gemm(routed_tile(M, K, false), direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
 
   // ---- dW_g = x_g^T g_g, contraction over the rows of group g ----
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]

@@ -100,6 +100,14 @@ FFNK_API size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N);
 FFNK_API int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t* out);
 
 /*
+ * Tuning hook: force every LDS-tiled GEMM launched by this process to use tile id `tile`
+ * (0 = 256x256 / 8 waves, 1 = 256x256 / 4 waves, 2 = 128x128 / 4 waves, 3 = small), or -1 to
+ * return to the tile table.  Process-global; meant for the tuner (python -m ffn_kernel_amd.tune),
+ * which plays the role of the reference's find_spec/*.py searches.  Returns the previous value.
+ */
+FFNK_API int ffnk_debug_force_tile(int tile);
+
+/*
  * MaskedLinear forward — replaces _bf16_linear_forward (ffn_kernel/linear.py:418-452):
  *   y[m, :] = x[m, :] @ (mask[m] ? Wv : Wt)      for m in [0, M)
  * x: [M, K], element strides (x_stride_m, 1).  Wv, Wt: logical [K, N] with element strides
