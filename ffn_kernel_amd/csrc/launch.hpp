@@ -66,6 +66,12 @@ int stream_chunk_k(int M, bool dual);         // K elements per streamed chunk
 int stream_waves_per_block(int M, bool dual); // wavefronts sharing one workgroup's K range
 hipError_t launch_stream_up(const StreamArgs& a, hipStream_t stream);
 hipError_t launch_stream_down(const StreamArgs& a, hipStream_t stream);
+// stream_dot.hip: M <= 8, contiguous-row dot-product kernels (splits == 1, P unused, no reduce pass).
+bool stream_dot_ok(int M, int K);
+int stream_dot_slices_per_wave(int K);
+int stream_dot_rows_per_block(int Nrows, bool dual, int K);
+hipError_t launch_stream_dot_up(const StreamArgs& a, hipStream_t stream);
+hipError_t launch_stream_dot_down(const StreamArgs& a, hipStream_t stream);
 // out[token row of p, n] = bf16(sum_s P[s][p][n])
 hipError_t launch_stream_reduce(const float* P, int splits, int M, int N, const uint8_t* mask, uint16_t* out,
                                 int64_t ldo, hipStream_t stream);

@@ -103,7 +103,7 @@ FFNK_API int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile
  * Tuning hook: force every LDS-tiled GEMM launched by this process to use tile id `tile`
  * (0 = 256x256 / 8 waves, 1 = 256x256 / 4 waves, 2 = 128x128 / 4 waves, 3 = small), or -1 to
  * return to the tile table.  Process-global; meant for the tuner (python -m ffn_kernel_amd.tune),
- * which plays the role of the reference's find_spec/*.py searches.  Returns the previous value.
+ * which plays the role of the reference's find_spec table lookups.  Returns the previous value.
  */
 FFNK_API int ffnk_debug_force_tile(int tile);
 

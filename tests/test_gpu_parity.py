@@ -220,6 +220,30 @@ def test_ffn_decode_path_vs_oracle(dev, M, kind, d, h):
         assert torch.equal(out2, out)
 
 
+# M <= 8 with K extents in whole 512-element slices: the contiguous-row dot-product streams
+DOT_SHAPES = [(1, "visual"), (1, "text"), (2, "bernoulli"), (3, "visual"), (4, "bernoulli"), (5, "text"),
+              (7, "bernoulli"), (8, "bernoulli"), (8, "visual")]
+
+
+@pytest.mark.parametrize("M,kind", DOT_SHAPES)
+@pytest.mark.parametrize("d,h", [(512, 1024), (1024, 4096), (4096, 1536), (1536, 7168)])
+def test_ffn_decode_dot_path_vs_oracle(dev, M, kind, d, h):
+    note(f"ffn decode dot M={M} kind={kind} d={d} h={h}")
+    cfg = _lib.tile_config(_lib.OP_FFN_UP, M, d, h)
+    assert cfg["path"] == _lib.PATH_STREAM and cfg["block_m"] == M and cfg["block_k"] in (512, 1024)
+    w = wl.cfg5_ffn_decode(M, kind, seed=40 + M, d=d, h=h)
+    w = wl.FFNWorkload(w.name, w.x, {k: (v.float() * 2.5).to(torch.bfloat16) for k, v in w.W.items()}, w.mask)
+    out = MaskedFFN.apply(*w.to(dev).op_args())
+    torch.cuda.synchronize()
+    assert_close(out, cref.ffn_fwd(w.x, w.W, w.mask, round_mid=True), f"decode dot {M} {kind}")
+    if kind in ("visual", "text"):
+        W = dict(w.W)
+        for k in (("u1", "u2", "u3") if kind == "visual" else ("w1", "w2", "w3")):
+            W[k] = torch.full_like(W[k], float("nan"))
+        out2 = MaskedFFN.apply(*wl.FFNWorkload("p", w.x, W, w.mask).to(dev).op_args())
+        assert torch.equal(out2, out)
+
+
 def test_ffn_decode_matches_tiled_path_rows(dev):
     """The same rows run as a decode call and inside a larger (tiled-path) call agree to bf16 accuracy."""
     note("ffn decode vs tiled")
