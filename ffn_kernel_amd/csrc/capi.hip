@@ -110,8 +110,14 @@ bool use_dot_path(int64_t M, int64_t d, int64_t h) {
   return use_stream_path(M, d, h) && stream_dot_ok((int)M, (int)d) && stream_dot_ok((int)M, (int)h);
 }
 
+// 9 <= M <= 64 (or smaller M whose extents the dot kernels do not take): LDS-transposed MFMA streams.
+bool use_tile_path(int64_t M, int64_t d, int64_t h) {
+  return use_stream_path(M, d, h) && !use_dot_path(M, d, h) && stream_tile_ok((int)M, (int)d, (int)h);
+}
+
 int down_splits(int64_t M, int64_t d, int64_t h) {
   if (use_dot_path(M, d, h)) return 1;
+  if (use_tile_path(M, d, h)) return stream_tile_down_splits((int)d, (int)h);
   return stream_down_splits(d, h, stream_rows_per_block((int)M, false), stream_waves_per_block((int)M, false));
 }
 
@@ -203,6 +209,13 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
     out->group_m = 1;
     out->split_k = stream_waves_per_block((int)M, up) * (up ? 1 : down_splits(M, K, N));
     out->direct_lds = 0;
+    if (use_tile_path(M, K, N)) {
+      // LDS-transposed streams: block_n weight rows (of each matrix) x 128-element chunks, three in flight
+      out->block_n = stream_tile_rows_per_block(up);
+      out->block_k = 128;
+      out->lds_stages = 3;
+      out->split_k = up ? 1 : down_splits(M, K, N);
+    }
     if (use_dot_path(M, K, N)) {
       // dot-product streams: a workgroup is block_n weight rows x all of K, one wavefront per
       // block_k-element slice of K
@@ -323,14 +336,17 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
     u.W0[0] = W1; u.W0[1] = U1; u.W1[0] = W3; u.W1[1] = U3; u.ldw = up_stride_n;
     u.Nrows = (int)h; u.K = (int)d; u.splits = 1; u.H = H; u.ldh = ldh; u.P = nullptr; u.out = nullptr; u.ldo = 0;
     const bool dot = use_dot_path(M, d, h);
-    FFNK_HIP(dot ? launch_stream_dot_up(u, stream) : launch_stream_up(u, stream), "streaming up-projection");
+    const bool tiled = use_tile_path(M, d, h);
+    FFNK_HIP(dot ? launch_stream_dot_up(u, stream) : tiled ? launch_stream_tile_up(u, stream) : launch_stream_up(u, stream),
+             "streaming up-projection");
     FFNK_HIP(mark(1), "event record");
     StreamArgs dn;
     dn.X = H; dn.ldx = ldh; dn.gather_x = 0; dn.mask = mask; dn.M = (int)M;
     dn.W0[0] = W2; dn.W0[1] = U2; dn.W1[0] = dn.W1[1] = nullptr; dn.ldw = down_stride_n;
     dn.Nrows = (int)d; dn.K = (int)h; dn.splits = splits; dn.H = nullptr; dn.ldh = 0;
     dn.P = splits > 1 ? P : nullptr; dn.out = out; dn.ldo = out_stride_m;
-    FFNK_HIP(dot ? launch_stream_dot_down(dn, stream) : launch_stream_down(dn, stream), "streaming down-projection");
+    FFNK_HIP(dot ? launch_stream_dot_down(dn, stream) : tiled ? launch_stream_tile_down(dn, stream) : launch_stream_down(dn, stream),
+             "streaming down-projection");
     if (splits > 1)
       FFNK_HIP(launch_stream_reduce(P, splits, (int)M, (int)d, mask, out, out_stride_m, stream), "streaming reduce");
     FFNK_HIP(mark(2), "event record");

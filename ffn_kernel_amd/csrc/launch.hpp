@@ -72,6 +72,12 @@ int stream_dot_slices_per_wave(int K);
 int stream_dot_rows_per_block(int Nrows, bool dual, int K);
 hipError_t launch_stream_dot_up(const StreamArgs& a, hipStream_t stream);
 hipError_t launch_stream_dot_down(const StreamArgs& a, hipStream_t stream);
+// stream_tile.hip: 9 <= M <= 64, contiguous loads + LDS transpose + shared token-row slab.
+bool stream_tile_ok(int M, int d, int h);
+int stream_tile_rows_per_block(bool dual);
+int stream_tile_down_splits(int d, int h);
+hipError_t launch_stream_tile_up(const StreamArgs& a, hipStream_t stream);
+hipError_t launch_stream_tile_down(const StreamArgs& a, hipStream_t stream);
 // out[token row of p, n] = bf16(sum_s P[s][p][n])
 hipError_t launch_stream_reduce(const float* P, int splits, int M, int N, const uint8_t* mask, uint16_t* out,
                                 int64_t ldo, hipStream_t stream);

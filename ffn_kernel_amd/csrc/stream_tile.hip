@@ -1,0 +1,279 @@
+// Weight-streaming MFMA kernels for decode-shaped MaskedFFN calls with 9 <= M <= 64 token rows.
+//
+// The op is bound by reading each present modality's weights once, and the MFMA operand layout
+// (lane = row, 16 bytes of K) would make every global load touch 16 rows x 64 bytes.  So the loads
+// are decoupled from that layout:
+//   * a wavefront owns two 16-row weight tiles (gate + up rows of the same outputs, or two row
+//     tiles of the down projection) and streams them in 128-element K chunks with loads that cover
+//     4 rows x 256 contiguous bytes each, kept three chunks (24 KB) ahead in registers;
+//   * each chunk is transposed through a wave-private, XOR-swizzled LDS tile (ds_write_b128 in load
+//     layout, ds_read_b128 in MFMA fragment layout, both bank-conflict free; one wavefront's LDS
+//     operations execute in order, so the tile needs neither double buffering nor waits);
+//   * the token rows of the chunk (x, or the SwiGLU intermediate) are staged once per workgroup in a
+//     double-buffered LDS slab that the four wavefronts share, fetched at the same distance as the
+//     weights so that the in-order load counter never forces a weight load to complete early;
+//   * one raw s_barrier per chunk hands the slab over; it does not drain the loads in flight.
+// The up projection covers all of K in one workgroup (SwiGLU epilogue, routed-order H); the down
+// projection splits K across workgroups into fp32 partials that stream_reduce_kernel sums.
+// Same role as the reference's small-M launches of its GEMM tiles (ffn_kernel/ffn.py:527-560,
+// ffn_kernel/linear.py:418-452).
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace ffnk {
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kTK = 128;    // K elements per chunk (16 pieces of 16 bytes per row)
+constexpr int kTD = 3;      // chunks in flight per wavefront
+constexpr int kTWaves = 4;  // wavefronts per workgroup
+constexpr int kTMaxM = 64;
+
+struct TileJob {
+  int grp, split, p0, mg, n0, c0, nc;  // n0: first weight row of the workgroup; c0 / nc: chunk range
+};
+
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes have landed
+  __builtin_amdgcn_s_barrier();
+}
+
+// xs: [2][NTM * 16 token rows][16 pieces] 16-byte slots; wst: this wavefront's [2 tiles][16 rows][16 pieces].
+template <int NTM, bool DUAL>
+__device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t, const int* s_perm, u32x4_t* xs,
+                                          u32x4_t* wst) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 15, lq = lane >> 4;
+  const int64_t kbase = (int64_t)t.c0 * kTK;
+
+  // weight tiles of this wavefront
+  int rbase[2];
+  const uint16_t* wp[2];
+  if (DUAL) {
+    rbase[0] = rbase[1] = t.n0 + wave * 16;
+    wp[0] = a.W0[t.grp];
+    wp[1] = a.W1[t.grp];
+  } else {
+    rbase[0] = t.n0 + wave * 32;
+    rbase[1] = rbase[0] + 16;
+    wp[0] = wp[1] = a.W0[t.grp];
+  }
+#pragma unroll
+  for (int w = 0; w < 2; ++w) wp[w] += (int64_t)(rbase[w] + lq) * a.ldw + kbase + lrow * 8;  // load u adds 4 u rows
+  const int64_t w_step = 4 * a.ldw;
+
+  // token-row pieces this thread stages: piece (tid & 15) of slab rows p * 16 + (tid >> 4)
+  const uint16_t* xp[NTM];
+#pragma unroll
+  for (int p = 0; p < NTM; ++p) {
+    const int j = p * 16 + (tid >> 4);
+    const int pos = t.p0 + min(j, t.mg - 1);  // surplus slab rows repeat the last row; dropped in the epilogue
+    const int64_t src = a.gather_x ? (int64_t)s_perm[pos] : (int64_t)pos;
+    xp[p] = a.X + src * a.ldx + kbase + (tid & 15) * 8;
+  }
+  const int x_slot = (tid >> 4) * 16 + ((tid & 15) ^ (tid >> 4));  // + p * 256: swizzled slab slot
+
+  u32x4_t wr[kTD][2][4];
+  u32x4_t xr[kTD][NTM];
+  auto loadw = [&](int s, int c) {
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        wr[s][w][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp[w] + u * w_step + (int64_t)c * kTK));
+  };
+  auto loadx = [&](int s, int c) {
+#pragma unroll
+    for (int p = 0; p < NTM; ++p) xr[s][p] = *reinterpret_cast<const u32x4_t*>(xp[p] + (int64_t)c * kTK);
+  };
+  auto stage_x = [&](int s, int c) {
+    u32x4_t* dst = xs + (c & 1) * (NTM * 256) + x_slot;
+#pragma unroll
+    for (int p = 0; p < NTM; ++p) dst[p * 256] = xr[s][p];
+  };
+
+  f32x4_t acc[2][NTM];
+#pragma unroll
+  for (int w = 0; w < 2; ++w)
+#pragma unroll
+    for (int m = 0; m < NTM; ++m) acc[w][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int nc = t.nc;
+  // prologue: chunks 0 .. kTD-1 of the weights, chunks 0 .. kTD of the token rows (chunk 0 goes
+  // straight to the slab), each only if it exists
+  loadx(0, 0);
+#pragma unroll
+  for (int s = 0; s < kTD; ++s) {
+    if (s < nc) loadw(s, s);
+    if (s >= 1 && s < nc) loadx(s, s);
+  }
+  stage_x(0, 0);
+  if (kTD < nc) loadx(0, kTD);
+  lds_barrier();
+
+  for (int c0 = 0; c0 < nc; c0 += kTD) {
+#pragma unroll
+    for (int u3 = 0; u3 < kTD; ++u3) {
+      const int c = c0 + u3;
+      if (c < nc) {
+        // weights of chunk c: registers -> swizzled staging tile
+#pragma unroll
+        for (int w = 0; w < 2; ++w)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int row = 4 * u + lq;
+            wst[w * 256 + row * 16 + (lrow ^ row)] = wr[u3][w][u];
+          }
+        if (c + kTD < nc) loadw(u3, c + kTD);
+        // token rows of chunk c + 1 -> the other slab buffer (its last readers passed the previous barrier)
+        if (c + 1 < nc) {
+          stage_x((u3 + 1) % kTD, c + 1);
+          if (c + 1 + kTD < nc) loadx((u3 + 1) % kTD, c + 1 + kTD);
+        }
+        const u32x4_t* xb = xs + (c & 1) * (NTM * 256);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const int piece = (s * 4 + lq) ^ lrow;
+          const bf16x8_t wf0 = __builtin_bit_cast(bf16x8_t, wst[lrow * 16 + piece]);
+          const bf16x8_t wf1 = __builtin_bit_cast(bf16x8_t, wst[256 + lrow * 16 + piece]);
+#pragma unroll
+          for (int m = 0; m < NTM; ++m) {
+            const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, xb[(m * 16 + lrow) * 16 + piece]);
+            acc[0][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, xf, acc[0][m], 0, 0, 0);
+            acc[1][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, xf, acc[1][m], 0, 0, 0);
+          }
+        }
+      }
+      lds_barrier();  // executed the same number of times by every wavefront (nc is uniform)
+    }
+  }
+
+  // acc[w][m][v]: weight row rbase[w] + 4 * lq + v, token row m * 16 + lrow of the group.
+#pragma unroll
+  for (int m = 0; m < NTM; ++m) {
+    const int row = m * 16 + lrow;
+    if (row >= t.mg) continue;
+    if (DUAL) {
+      const f32x4_t g = acc[0][m], u = acc[1][m];
+      uint2 v2;
+      v2.x = pack2bf(swiglu(g[0], u[0]), swiglu(g[1], u[1]));
+      v2.y = pack2bf(swiglu(g[2], u[2]), swiglu(g[3], u[3]));
+      *reinterpret_cast<uint2*>(a.H + (int64_t)(t.p0 + row) * a.ldh + rbase[0] + 4 * lq) = v2;
+    } else {
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const f32x4_t o = acc[w][m];
+        const int n_out = rbase[w] + 4 * lq;
+        if (a.P != nullptr) {
+          *reinterpret_cast<float4*>(a.P + ((int64_t)t.split * a.M + (t.p0 + row)) * a.Nrows + n_out) =
+              make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+          uint16_t* dst = a.out + (int64_t)s_perm[t.p0 + row] * a.ldo + n_out;
+          if ((reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+            uint2 v2;
+            v2.x = pack2bf(o[0], o[1]);
+            v2.y = pack2bf(o[2], o[3]);
+            *reinterpret_cast<uint2*>(dst) = v2;
+          } else {
+            dst[0] = f2bf(o[0]); dst[1] = f2bf(o[1]); dst[2] = f2bf(o[2]); dst[3] = f2bf(o[3]);
+          }
+        }
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ int route64(const uint8_t* mask, int M, int* s_perm, int* s_nvis) {
+  if (threadIdx.x < kWave) {
+    const int l = threadIdx.x;
+    const bool valid = l < M;
+    const bool vis = valid && mask[l] != 0;
+    const unsigned long long vm = __ballot(vis);
+    const unsigned long long am = __ballot(valid);
+    const unsigned long long lt = (l == 0) ? 0ull : (~0ull >> (64 - l));
+    const int nv = __popcll(vm);
+    if (valid) s_perm[vis ? __popcll(vm & lt) : nv + __popcll(~vm & am & lt)] = l;
+    if (l == 0) *s_nvis = nv;
+  }
+  __syncthreads();
+  return *s_nvis;
+}
+
+// grid.x = 2 groups x splits x row blocks (visual workgroups first); 256 threads.
+template <int NTM_MAX, bool DUAL>
+__global__ __launch_bounds__(kTWaves * kWave, 2) void stream_tile_kernel(const StreamArgs a) {
+  __shared__ u32x4_t xs[2 * NTM_MAX * 256];
+  __shared__ u32x4_t wst_all[kTWaves * 512];
+  __shared__ int s_perm[kTMaxM];
+  __shared__ int s_nvis;
+  const int n_vis = route64(a.mask, a.M, s_perm, &s_nvis);
+  constexpr int ROWS = DUAL ? 16 * kTWaves : 32 * kTWaves;
+  const int row_blocks = a.Nrows / ROWS;
+  const int per_grp = row_blocks * a.splits;
+  TileJob t;
+  t.grp = blockIdx.x / per_grp;
+  const int rem = blockIdx.x % per_grp;
+  t.split = rem / row_blocks;
+  t.p0 = t.grp == 0 ? 0 : n_vis;
+  t.mg = t.grp == 0 ? n_vis : a.M - n_vis;
+  if (t.mg == 0) return;  // modality absent: its weights are never read (uniform over the workgroup)
+  t.n0 = (rem % row_blocks) * ROWS;
+  const int n_chunks = a.K / kTK;
+  const int cps = cdiv(n_chunks, a.splits);
+  t.c0 = min(t.split * cps, n_chunks);
+  t.nc = min(t.c0 + cps, n_chunks) - t.c0;
+  u32x4_t* wst = wst_all + (threadIdx.x >> 6) * 512;
+  const int ntm = cdiv(t.mg, 16);
+  if (NTM_MAX >= 4 && ntm >= 4) tile_rows<(NTM_MAX >= 4 ? 4 : 1), DUAL>(a, t, s_perm, xs, wst);
+  else if (NTM_MAX >= 3 && ntm == 3) tile_rows<(NTM_MAX >= 3 ? 3 : 1), DUAL>(a, t, s_perm, xs, wst);
+  else if (NTM_MAX >= 2 && ntm == 2) tile_rows<(NTM_MAX >= 2 ? 2 : 1), DUAL>(a, t, s_perm, xs, wst);
+  else tile_rows<1, DUAL>(a, t, s_perm, xs, wst);
+}
+
+int stream_tile_rows_per_block(bool dual) { return dual ? 16 * kTWaves : 32 * kTWaves; }
+
+bool stream_tile_ok(int M, int d, int h) {
+  return M >= 1 && M <= kTMaxM && d % kTK == 0 && h % kTK == 0 && h % stream_tile_rows_per_block(true) == 0 &&
+         d % stream_tile_rows_per_block(false) == 0;
+}
+
+// K split of the down projection: about one workgroup per CU and modality, at least eight chunks
+// per workgroup, every split non-empty.
+int stream_tile_down_splits(int d, int h) {
+  const int row_blocks = d / stream_tile_rows_per_block(false);
+  const int n_chunks = h / kTK;
+  int s = cdiv(256, row_blocks);
+  if (s > n_chunks / 8) s = n_chunks / 8;
+  if (s < 1) s = 1;
+  while (s > 1 && cdiv(n_chunks, s) * (s - 1) >= n_chunks) --s;  // last split would be empty
+  return s;
+}
+
+template <int NTM_MAX, bool DUAL>
+static void launch_tile_n(const StreamArgs& a, hipStream_t stream) {
+  const int blocks = 2 * (a.Nrows / stream_tile_rows_per_block(DUAL)) * a.splits;
+  hipLaunchKernelGGL((stream_tile_kernel<NTM_MAX, DUAL>), dim3(blocks), dim3(kTWaves * kWave), 0, stream, a);
+}
+
+template <bool DUAL>
+static hipError_t launch_tile(const StreamArgs& a, hipStream_t stream) {
+  if (a.M < 1 || a.M > kTMaxM || a.K % kTK != 0 || a.splits < 1 || a.Nrows % stream_tile_rows_per_block(DUAL) != 0 ||
+      a.ldw % 8 != 0 || a.ldx % 8 != 0)
+    return hipErrorInvalidValue;
+  const int n_chunks = a.K / kTK;
+  if (cdiv(n_chunks, a.splits) * (a.splits - 1) >= n_chunks) return hipErrorInvalidValue;  // an empty split
+  if (DUAL && (a.splits != 1 || a.H == nullptr)) return hipErrorInvalidValue;
+  if (!DUAL && a.P == nullptr && (a.splits != 1 || a.out == nullptr)) return hipErrorInvalidValue;
+  switch (cdiv(a.M, 16)) {
+    case 1: launch_tile_n<1, DUAL>(a, stream); break;
+    case 2: launch_tile_n<2, DUAL>(a, stream); break;
+    case 3: launch_tile_n<3, DUAL>(a, stream); break;
+    default: launch_tile_n<4, DUAL>(a, stream); break;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_stream_tile_up(const StreamArgs& a, hipStream_t stream) { return launch_tile<true>(a, stream); }
+hipError_t launch_stream_tile_down(const StreamArgs& a, hipStream_t stream) { return launch_tile<false>(a, stream); }
+
+}  // namespace ffnk

@@ -42,9 +42,19 @@ def test_tile_table_entries():
     big = _lib.tile_config(_lib.OP_FFN_UP, 32768, 4096, 14336)
     assert big["path"] == _lib.PATH_MFMA_TILED and big["block_m"] == 256 and big["direct_lds"] == 1
     assert big["block_k"] == 32 and big["lds_stages"] == 4  # direct global->LDS ring
+    # M <= 8: dot-product streams, one wavefront per 1024-element K slice, no cross-workgroup split
     dec = _lib.tile_config(_lib.OP_FFN_FWD, 8, 4096, 14336)
-    assert dec["path"] == _lib.PATH_STREAM and dec["lds_stages"] == 0 and dec["block_m"] == 16
+    assert dec["path"] == _lib.PATH_STREAM and dec["lds_stages"] == 0 and dec["block_m"] == 8
+    assert dec["block_k"] == 1024 and dec["split_k"] == 4
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 8, 4096, 14336)["split_k"] == 14
+    # 9 <= M <= 64: LDS-transposed streams, 128-element chunks, three in flight, split-K down projection
+    mid = _lib.tile_config(_lib.OP_FFN_UP, 64, 4096, 14336)
+    assert mid["path"] == _lib.PATH_STREAM and mid["block_k"] == 128 and mid["lds_stages"] == 3
+    assert mid["block_n"] == 64 and mid["split_k"] == 1
     assert _lib.tile_config(_lib.OP_FFN_DOWN, 64, 4096, 14336)["split_k"] >= 4
+    # small M whose extents are not whole 512-element slices run on the LDS-transposed streams too
+    odd = _lib.tile_config(_lib.OP_FFN_UP, 4, 384, 640)
+    assert odd["path"] == _lib.PATH_STREAM and odd["lds_stages"] == 3
     assert _lib.tile_config(_lib.OP_FFN_FWD, 65, 4096, 14336)["path"] == _lib.PATH_MFMA_TILED
     small = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 1024, 1024)
     assert small["block_m"] * small["block_n"] < 256 * 256  # small problems get small tiles
