@@ -117,7 +117,7 @@ bool use_tile_path(int64_t M, int64_t d, int64_t h) {
 
 int down_splits(int64_t M, int64_t d, int64_t h) {
   if (use_dot_path(M, d, h)) return 1;
-  if (use_tile_path(M, d, h)) return stream_tile_down_splits((int)d, (int)h);
+  if (use_tile_path(M, d, h)) return stream_tile_down_splits((int)M, (int)d, (int)h);
   return stream_down_splits(d, h, stream_rows_per_block((int)M, false), stream_waves_per_block((int)M, false));
 }
 
@@ -211,9 +211,9 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
     out->direct_lds = 0;
     if (use_tile_path(M, K, N)) {
       // LDS-transposed streams: block_n weight rows (of each matrix) x 128-element chunks, three in flight
-      out->block_n = stream_tile_rows_per_block(up);
+      out->block_n = stream_tile_rows_per_block((int)M, up);
       out->block_k = 128;
-      out->lds_stages = 3;
+      out->lds_stages = stream_tile_depth((int)M);
       out->split_k = up ? 1 : down_splits(M, K, N);
     }
     if (use_dot_path(M, K, N)) {

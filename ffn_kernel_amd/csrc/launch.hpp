@@ -74,8 +74,9 @@ hipError_t launch_stream_dot_up(const StreamArgs& a, hipStream_t stream);
 hipError_t launch_stream_dot_down(const StreamArgs& a, hipStream_t stream);
 // stream_tile.hip: 9 <= M <= 64, contiguous loads + LDS transpose + shared token-row slab.
 bool stream_tile_ok(int M, int d, int h);
-int stream_tile_rows_per_block(bool dual);
-int stream_tile_down_splits(int d, int h);
+int stream_tile_rows_per_block(int M, bool dual);
+int stream_tile_depth(int M);
+int stream_tile_down_splits(int M, int d, int h);
 hipError_t launch_stream_tile_up(const StreamArgs& a, hipStream_t stream);
 hipError_t launch_stream_tile_down(const StreamArgs& a, hipStream_t stream);
 // out[token row of p, n] = bf16(sum_s P[s][p][n])

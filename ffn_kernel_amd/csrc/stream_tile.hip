@@ -5,18 +5,20 @@
 // are decoupled from that layout:
 //   * a wavefront owns two 16-row weight tiles (gate + up rows of the same outputs, or two row
 //     tiles of the down projection) and streams them in 128-element K chunks with loads that cover
-//     4 rows x 256 contiguous bytes each, kept three chunks (24 KB) ahead in registers;
+//     4 rows x 256 contiguous bytes each, kept three or four chunks (24-32 KB) ahead in registers;
 //   * each chunk is transposed through a wave-private, XOR-swizzled LDS tile (ds_write_b128 in load
 //     layout, ds_read_b128 in MFMA fragment layout, both bank-conflict free; one wavefront's LDS
 //     operations execute in order, so the tile needs neither double buffering nor waits);
 //   * the token rows of the chunk (x, or the SwiGLU intermediate) are staged once per workgroup in a
-//     double-buffered LDS slab that the four wavefronts share, fetched at the same distance as the
+//     double-buffered LDS slab that the wavefronts of the workgroup share, fetched at the same distance as the
 //     weights so that the in-order load counter never forces a weight load to complete early;
 //   * one raw s_barrier per chunk hands the slab over; it does not drain the loads in flight.
 // The up projection covers all of K in one workgroup (SwiGLU epilogue, routed-order H); the down
 // projection splits K across workgroups into fp32 partials that stream_reduce_kernel sums.
 // Same role as the reference's small-M launches of its GEMM tiles (ffn_kernel/ffn.py:527-560,
 // ffn_kernel/linear.py:418-452).
+#include <type_traits>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -25,21 +27,22 @@ namespace ffnk {
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kTK = 128;    // K elements per chunk (16 pieces of 16 bytes per row)
-constexpr int kTD = 3;      // chunks in flight per wavefront
-constexpr int kTWaves = 4;  // wavefronts per workgroup
+// Shape per number of 16-row m-tiles the call can have (ceil(M / 16)): wavefronts per workgroup
+// (sharing one token-row slab; fewer wavefronts = less barrier coupling and more workgroups, but
+// every thread then stages more of the slab) and chunks in flight per wavefront (register budget).
+#ifndef FFNK_TILE_SHAPES
+#define FFNK_TILE_SHAPES {2, 4}, {2, 3}, {4, 3}, {4, 3}
+#endif
+struct TileShapeEntry { int waves, depth; };
+constexpr TileShapeEntry kTileShapes[4] = {FFNK_TILE_SHAPES};
 constexpr int kTMaxM = 64;
 
 struct TileJob {
   int grp, split, p0, mg, n0, c0, nc;  // n0: first weight row of the workgroup; c0 / nc: chunk range
 };
 
-__device__ __forceinline__ void lds_barrier() {
-  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes have landed
-  __builtin_amdgcn_s_barrier();
-}
-
 // xs: [2][NTM * 16 token rows][16 pieces] 16-byte slots; wst: this wavefront's [2 tiles][16 rows][16 pieces].
-template <int NTM, bool DUAL>
+template <int NTM, bool DUAL, int kTWaves, int kTD>
 __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t, const int* s_perm, u32x4_t* xs,
                                           u32x4_t* wst) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -62,34 +65,51 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
   for (int w = 0; w < 2; ++w) wp[w] += (int64_t)(rbase[w] + lq) * a.ldw + kbase + lrow * 8;  // load u adds 4 u rows
   const int64_t w_step = 4 * a.ldw;
 
-  // token-row pieces this thread stages: piece (tid & 15) of slab rows p * 16 + (tid >> 4)
-  const uint16_t* xp[NTM];
+  // Token-row slab: two buffers of [NTM * 16 rows][16 pieces].  Each thread stages piece (tid & 15)
+  // of slab rows p * XR + (tid >> 4); slot = row * 16 + (piece ^ row & 15).
+  constexpr int XR = kTWaves * 4;    // slab rows one pass of the workgroup covers
+  constexpr int XP = NTM * 16 / XR;  // passes
+  const uint16_t* xp[XP];
 #pragma unroll
-  for (int p = 0; p < NTM; ++p) {
-    const int j = p * 16 + (tid >> 4);
+  for (int p = 0; p < XP; ++p) {
+    const int j = p * XR + (tid >> 4);
     const int pos = t.p0 + min(j, t.mg - 1);  // surplus slab rows repeat the last row; dropped in the epilogue
     const int64_t src = a.gather_x ? (int64_t)s_perm[pos] : (int64_t)pos;
     xp[p] = a.X + src * a.ldx + kbase + (tid & 15) * 8;
   }
-  const int x_slot = (tid >> 4) * 16 + ((tid & 15) ^ (tid >> 4));  // + p * 256: swizzled slab slot
 
+  // Workgroups walk their chunk range from different starting chunks (wrapping around): weight rows
+  // are a power-of-two number of bytes apart, so workgroups sitting at the same K offset would all
+  // pull from the same few HBM channels.
+  const int nc = t.nc;
+  const int rot = (int)((blockIdx.x * 11u) % (unsigned)nc);
+  auto phys = [&](int c) { const int pc = c + rot; return (pc >= nc ? pc - nc : pc) * kTK; };
   u32x4_t wr[kTD][2][4];
-  u32x4_t xr[kTD][NTM];
   auto loadw = [&](int s, int c) {
+    const int64_t ko = phys(c);
 #pragma unroll
     for (int w = 0; w < 2; ++w)
 #pragma unroll
       for (int u = 0; u < 4; ++u)
-        wr[s][w][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp[w] + u * w_step + (int64_t)c * kTK));
+        wr[s][w][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp[w] + u * w_step + ko));
   };
+  u32x4_t xr[kTD][XP];
   auto loadx = [&](int s, int c) {
+    const int64_t ko = phys(c);
 #pragma unroll
-    for (int p = 0; p < NTM; ++p) xr[s][p] = *reinterpret_cast<const u32x4_t*>(xp[p] + (int64_t)c * kTK);
+    for (int p = 0; p < XP; ++p) xr[s][p] = *reinterpret_cast<const u32x4_t*>(xp[p] + ko);
   };
   auto stage_x = [&](int s, int c) {
-    u32x4_t* dst = xs + (c & 1) * (NTM * 256) + x_slot;
+    u32x4_t* dst = xs + (c & 1) * (NTM * 256);
 #pragma unroll
-    for (int p = 0; p < NTM; ++p) dst[p * 256] = xr[s][p];
+    for (int p = 0; p < XP; ++p) {
+      const int j = p * XR + (tid >> 4);
+      dst[j * 16 + ((tid & 15) ^ (j & 15))] = xr[s][p];
+    }
+  };
+  auto lds_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes have landed; loads stay in flight
+    __builtin_amdgcn_s_barrier();
   };
 
   f32x4_t acc[2][NTM];
@@ -98,53 +118,64 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
 #pragma unroll
     for (int m = 0; m < NTM; ++m) acc[w][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int nc = t.nc;
-  // prologue: chunks 0 .. kTD-1 of the weights, chunks 0 .. kTD of the token rows (chunk 0 goes
-  // straight to the slab), each only if it exists
+  // One chunk.  STEADY: chunk c + 1 + kTD exists, so every load below is issued unconditionally and
+  // the compiler's load-counter waits are exact; otherwise the loads are guarded, which makes the
+  // compiler wait for more than it needs - only the last 2 kTD chunks of a workgroup run that way.
+  // Loads go out as w(c + kTD), x(c + 1 + kTD): the token rows of a chunk are fetched at the same
+  // distance as its weights, so waiting for them never forces younger weight loads to land.
+  auto chunk = [&](int u3, int c, auto steady_tag) {
+    constexpr bool STEADY = decltype(steady_tag)::value;
+    // weights of chunk c: registers -> swizzled staging tile
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int row = 4 * u + lq;
+        wst[w * 256 + row * 16 + (lrow ^ row)] = wr[u3][w][u];
+      }
+    if (STEADY || c + kTD < nc) loadw(u3, c + kTD);
+    // token rows of chunk c + 1 -> the other slab buffer (its last readers passed the previous barrier)
+    if (STEADY || c + 1 < nc) {
+      stage_x((u3 + 1) % kTD, c + 1);
+      if (STEADY || c + 1 + kTD < nc) loadx((u3 + 1) % kTD, c + 1 + kTD);
+    }
+    const u32x4_t* xb = xs + (c & 1) * (NTM * 256);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int piece = (s * 4 + lq) ^ lrow;
+      const bf16x8_t wf0 = __builtin_bit_cast(bf16x8_t, wst[lrow * 16 + piece]);
+      const bf16x8_t wf1 = __builtin_bit_cast(bf16x8_t, wst[256 + lrow * 16 + piece]);
+#pragma unroll
+      for (int m = 0; m < NTM; ++m) {
+        const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, xb[(m * 16 + lrow) * 16 + piece]);
+        acc[0][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, xf, acc[0][m], 0, 0, 0);
+        acc[1][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, xf, acc[1][m], 0, 0, 0);
+      }
+    }
+    lds_barrier();  // executed the same number of times by every wavefront (nc is uniform)
+  };
+
+  // prologue (nc >= 2 kTD, checked on the host): weights of chunks 0 .. kTD-1, token rows of chunks
+  // 0 .. kTD; chunk 0's go straight to the slab
   loadx(0, 0);
 #pragma unroll
   for (int s = 0; s < kTD; ++s) {
-    if (s < nc) loadw(s, s);
-    if (s >= 1 && s < nc) loadx(s, s);
+    loadw(s, s);
+    if (s >= 1) loadx(s, s);
   }
   stage_x(0, 0);
-  if (kTD < nc) loadx(0, kTD);
+  loadx(0, kTD);
   lds_barrier();
 
-  for (int c0 = 0; c0 < nc; c0 += kTD) {
+  int c0 = 0;
+  for (; c0 + 2 * kTD < nc; c0 += kTD) {
+#pragma unroll
+    for (int u3 = 0; u3 < kTD; ++u3) chunk(u3, c0 + u3, std::true_type{});
+  }
+  for (; c0 < nc; c0 += kTD) {
 #pragma unroll
     for (int u3 = 0; u3 < kTD; ++u3) {
-      const int c = c0 + u3;
-      if (c < nc) {
-        // weights of chunk c: registers -> swizzled staging tile
-#pragma unroll
-        for (int w = 0; w < 2; ++w)
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const int row = 4 * u + lq;
-            wst[w * 256 + row * 16 + (lrow ^ row)] = wr[u3][w][u];
-          }
-        if (c + kTD < nc) loadw(u3, c + kTD);
-        // token rows of chunk c + 1 -> the other slab buffer (its last readers passed the previous barrier)
-        if (c + 1 < nc) {
-          stage_x((u3 + 1) % kTD, c + 1);
-          if (c + 1 + kTD < nc) loadx((u3 + 1) % kTD, c + 1 + kTD);
-        }
-        const u32x4_t* xb = xs + (c & 1) * (NTM * 256);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const int piece = (s * 4 + lq) ^ lrow;
-          const bf16x8_t wf0 = __builtin_bit_cast(bf16x8_t, wst[lrow * 16 + piece]);
-          const bf16x8_t wf1 = __builtin_bit_cast(bf16x8_t, wst[256 + lrow * 16 + piece]);
-#pragma unroll
-          for (int m = 0; m < NTM; ++m) {
-            const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, xb[(m * 16 + lrow) * 16 + piece]);
-            acc[0][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, xf, acc[0][m], 0, 0, 0);
-            acc[1][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, xf, acc[1][m], 0, 0, 0);
-          }
-        }
-      }
-      lds_barrier();  // executed the same number of times by every wavefront (nc is uniform)
+      if (c0 + u3 < nc) chunk(u3, c0 + u3, std::false_type{});  // uniform over the workgroup
     }
   }
 
@@ -200,7 +231,7 @@ __device__ __forceinline__ int route64(const uint8_t* mask, int M, int* s_perm, 
 }
 
 // grid.x = 2 groups x splits x row blocks (visual workgroups first); 256 threads.
-template <int NTM_MAX, bool DUAL>
+template <int NTM_MAX, bool DUAL, int kTWaves, int kTD>
 __global__ __launch_bounds__(kTWaves * kWave, 2) void stream_tile_kernel(const StreamArgs a) {
   __shared__ u32x4_t xs[2 * NTM_MAX * 256];
   __shared__ u32x4_t wst_all[kTWaves * 512];
@@ -224,44 +255,51 @@ __global__ __launch_bounds__(kTWaves * kWave, 2) void stream_tile_kernel(const S
   t.nc = min(t.c0 + cps, n_chunks) - t.c0;
   u32x4_t* wst = wst_all + (threadIdx.x >> 6) * 512;
   const int ntm = cdiv(t.mg, 16);
-  if (NTM_MAX >= 4 && ntm >= 4) tile_rows<(NTM_MAX >= 4 ? 4 : 1), DUAL>(a, t, s_perm, xs, wst);
-  else if (NTM_MAX >= 3 && ntm == 3) tile_rows<(NTM_MAX >= 3 ? 3 : 1), DUAL>(a, t, s_perm, xs, wst);
-  else if (NTM_MAX >= 2 && ntm == 2) tile_rows<(NTM_MAX >= 2 ? 2 : 1), DUAL>(a, t, s_perm, xs, wst);
-  else tile_rows<1, DUAL>(a, t, s_perm, xs, wst);
+  if (NTM_MAX >= 4 && ntm >= 4) tile_rows<(NTM_MAX >= 4 ? 4 : 1), DUAL, kTWaves, kTD>(a, t, s_perm, xs, wst);
+  else if (NTM_MAX >= 3 && ntm == 3) tile_rows<(NTM_MAX >= 3 ? 3 : 1), DUAL, kTWaves, kTD>(a, t, s_perm, xs, wst);
+  else if (NTM_MAX >= 2 && ntm == 2) tile_rows<(NTM_MAX >= 2 ? 2 : 1), DUAL, kTWaves, kTD>(a, t, s_perm, xs, wst);
+  else tile_rows<1, DUAL, kTWaves, kTD>(a, t, s_perm, xs, wst);
 }
 
-int stream_tile_rows_per_block(bool dual) { return dual ? 16 * kTWaves : 32 * kTWaves; }
+static int tile_waves(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].waves; }
+
+int stream_tile_rows_per_block(int M, bool dual) { return (dual ? 16 : 32) * tile_waves(M); }
+int stream_tile_depth(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].depth; }
+
+constexpr int kTMinChunks = 8;  // >= 2 x the deepest ring: lets the kernels run an unconditional prologue
 
 bool stream_tile_ok(int M, int d, int h) {
-  return M >= 1 && M <= kTMaxM && d % kTK == 0 && h % kTK == 0 && h % stream_tile_rows_per_block(true) == 0 &&
-         d % stream_tile_rows_per_block(false) == 0;
+  return M >= 1 && M <= kTMaxM && d % kTK == 0 && h % kTK == 0 && d / kTK >= kTMinChunks && h / kTK >= kTMinChunks &&
+         h % stream_tile_rows_per_block(M, true) == 0 && d % stream_tile_rows_per_block(M, false) == 0;
 }
 
 // K split of the down projection: about one workgroup per CU and modality, at least eight chunks
 // per workgroup, every split non-empty.
-int stream_tile_down_splits(int d, int h) {
-  const int row_blocks = d / stream_tile_rows_per_block(false);
+int stream_tile_down_splits(int M, int d, int h) {
+  const int row_blocks = d / stream_tile_rows_per_block(M, false);
   const int n_chunks = h / kTK;
   int s = cdiv(256, row_blocks);
-  if (s > n_chunks / 8) s = n_chunks / 8;
+  if (s > n_chunks / kTMinChunks) s = n_chunks / kTMinChunks;
   if (s < 1) s = 1;
-  while (s > 1 && cdiv(n_chunks, s) * (s - 1) >= n_chunks) --s;  // last split would be empty
+  // every split must keep at least kTMinChunks chunks (the last one gets the remainder)
+  while (s > 1 && n_chunks - cdiv(n_chunks, s) * (s - 1) < kTMinChunks) --s;
   return s;
 }
 
 template <int NTM_MAX, bool DUAL>
 static void launch_tile_n(const StreamArgs& a, hipStream_t stream) {
-  const int blocks = 2 * (a.Nrows / stream_tile_rows_per_block(DUAL)) * a.splits;
-  hipLaunchKernelGGL((stream_tile_kernel<NTM_MAX, DUAL>), dim3(blocks), dim3(kTWaves * kWave), 0, stream, a);
+  constexpr int W = kTileShapes[NTM_MAX - 1].waves, D = kTileShapes[NTM_MAX - 1].depth;
+  const int blocks = 2 * (a.Nrows / ((DUAL ? 16 : 32) * W)) * a.splits;
+  hipLaunchKernelGGL((stream_tile_kernel<NTM_MAX, DUAL, W, D>), dim3(blocks), dim3(W * kWave), 0, stream, a);
 }
 
 template <bool DUAL>
 static hipError_t launch_tile(const StreamArgs& a, hipStream_t stream) {
-  if (a.M < 1 || a.M > kTMaxM || a.K % kTK != 0 || a.splits < 1 || a.Nrows % stream_tile_rows_per_block(DUAL) != 0 ||
+  if (a.M < 1 || a.M > kTMaxM || a.K % kTK != 0 || a.splits < 1 || a.Nrows % stream_tile_rows_per_block(a.M, DUAL) != 0 ||
       a.ldw % 8 != 0 || a.ldx % 8 != 0)
     return hipErrorInvalidValue;
   const int n_chunks = a.K / kTK;
-  if (cdiv(n_chunks, a.splits) * (a.splits - 1) >= n_chunks) return hipErrorInvalidValue;  // an empty split
+  if (n_chunks - cdiv(n_chunks, a.splits) * (a.splits - 1) < kTMinChunks) return hipErrorInvalidValue;  // a short split
   if (DUAL && (a.splits != 1 || a.H == nullptr)) return hipErrorInvalidValue;
   if (!DUAL && a.P == nullptr && (a.splits != 1 || a.out == nullptr)) return hipErrorInvalidValue;
   switch (cdiv(a.M, 16)) {

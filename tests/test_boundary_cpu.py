@@ -52,9 +52,13 @@ def test_tile_table_entries():
     assert mid["path"] == _lib.PATH_STREAM and mid["block_k"] == 128 and mid["lds_stages"] == 3
     assert mid["block_n"] == 64 and mid["split_k"] == 1
     assert _lib.tile_config(_lib.OP_FFN_DOWN, 64, 4096, 14336)["split_k"] >= 4
-    # small M whose extents are not whole 512-element slices run on the LDS-transposed streams too
-    odd = _lib.tile_config(_lib.OP_FFN_UP, 4, 384, 640)
-    assert odd["path"] == _lib.PATH_STREAM and odd["lds_stages"] == 3
+    assert _lib.tile_config(_lib.OP_FFN_UP, 16, 4096, 14336)["block_n"] == 32  # two wavefronts per workgroup
+    # small M whose extents are not whole 512-element slices run on the LDS-transposed streams too ...
+    odd = _lib.tile_config(_lib.OP_FFN_UP, 4, 1152, 1408)
+    assert odd["path"] == _lib.PATH_STREAM and odd["lds_stages"] >= 3
+    # ... and extents under 1024 on the fragment-layout streams
+    tiny = _lib.tile_config(_lib.OP_FFN_UP, 4, 384, 640)
+    assert tiny["path"] == _lib.PATH_STREAM and tiny["lds_stages"] == 0
     assert _lib.tile_config(_lib.OP_FFN_FWD, 65, 4096, 14336)["path"] == _lib.PATH_MFMA_TILED
     small = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 1024, 1024)
     assert small["block_m"] * small["block_n"] < 256 * 256  # small problems get small tiles

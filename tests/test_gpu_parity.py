@@ -244,6 +244,32 @@ def test_ffn_decode_dot_path_vs_oracle(dev, M, kind, d, h):
         assert torch.equal(out2, out)
 
 
+# 9 <= M <= 64 (and smaller M off the dot kernels' extents) with d, h >= 1024: LDS-transposed streams
+TILE_STREAM_SHAPES = [(9, "bernoulli"), (16, "visual"), (17, "bernoulli"), (31, "text"), (33, "text"),
+                      (48, "bernoulli"), (64, "bernoulli"), (64, "visual"), (5, "bernoulli")]
+
+
+@pytest.mark.parametrize("M,kind", TILE_STREAM_SHAPES)
+@pytest.mark.parametrize("d,h", [(1024, 2048), (2048, 1024), (1152, 1408)])
+def test_ffn_decode_tile_stream_vs_oracle(dev, M, kind, d, h):
+    note(f"ffn decode tile stream M={M} kind={kind} d={d} h={h}")
+    cfg = _lib.tile_config(_lib.OP_FFN_UP, M, d, h)
+    assert cfg["path"] == _lib.PATH_STREAM
+    if M > 8 or d % 512:
+        assert cfg["block_k"] == 128 and cfg["lds_stages"] >= 3
+    w = wl.cfg5_ffn_decode(M, kind, seed=70 + M, d=d, h=h)
+    w = wl.FFNWorkload(w.name, w.x, {k: (v.float() * 1.5).to(torch.bfloat16) for k, v in w.W.items()}, w.mask)
+    out = MaskedFFN.apply(*w.to(dev).op_args())
+    torch.cuda.synchronize()
+    assert_close(out, cref.ffn_fwd(w.x, w.W, w.mask, round_mid=True), f"decode tile stream {M} {kind}")
+    if kind in ("visual", "text"):
+        W = dict(w.W)
+        for k in (("u1", "u2", "u3") if kind == "visual" else ("w1", "w2", "w3")):
+            W[k] = torch.full_like(W[k], float("nan"))
+        out2 = MaskedFFN.apply(*wl.FFNWorkload("p", w.x, W, w.mask).to(dev).op_args())
+        assert torch.equal(out2, out)
+
+
 def test_ffn_decode_matches_tiled_path_rows(dev):
     """The same rows run as a decode call and inside a larger (tiled-path) call agree to bf16 accuracy."""
     note("ffn decode vs tiled")
