@@ -26,12 +26,15 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (KiB per dispatch, scaled by what the same counters read for the 1 GiB copy of --workload copy1g:
 # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  The counter runs and the arithmetic are kept as text under
-# profiles/ (routed_gemm_kernel_ffn_fwd_M32768_d4096_h14336.txt, stream_kernel_ffn_decode_*.txt).
+# profiles/ (routed_gemm_kernel_ffn_fwd_M32768_d4096_h14336.txt, stream_*_kernel_ffn_decode_*.txt).
 # Recorded, not measured live: counters cannot be read from inside the process.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg4": (8.3811e6 * 2.0 + 9.2594e5) * 1024,                       # up-projection kernel
-    "decode8": (2.4124e5 * 2.0 + 224 + 1.19e5 * 2.0 + 64) * 1024,     # both stream kernels of a call
-    "decode1v": (1.2051e5 * 2.0 + 28 + 5.9402e4 * 2.0 + 8) * 1024,
+    "cfg4": (8.3811e6 * 2.0 + 9.2594e5) * 1024,                                   # up-projection kernel
+    # decode: all launches of one call (up-projection, down-projection, reduce where there is one)
+    "decode1v": (1.1476e5 * 2.0 + 40 + 5.7481e4 * 2.0 + 8) * 1024,
+    "decode8": (2.2979e5 * 2.0 + 320 + 1.1568e5 * 2.0 + 64) * 1024,
+    "decode32": (2.3053e5 * 2.0 + 896 + 1.184e5 * 2.0 + 2048 + 1039 * 2.0 + 256) * 1024,
+    "decode64": (2.3159e5 * 2.0 + 1792 + 1.2202e5 * 2.0 + 8193 + 4111 * 2.0 + 512) * 1024,
 }
 
 
@@ -205,7 +208,7 @@ def main() -> int:
         achieved = call_bytes / (ms_per_step * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": achieved / PEAK_HBM_GBS, "traffic": traffic,
-                    "kernel": "stream_kernel x2 (up-projection + SwiGLU, down-projection)",
+                    "kernel": "decode stream kernels of one call (up-projection + SwiGLU, down-projection)",
                     "kernel_ms": ms_per_step, "algorithmic_bytes": call_bytes,
                     "up_ms_with_event_gap": up_avg, "down_ms_with_event_gap": down_avg}
     else:
