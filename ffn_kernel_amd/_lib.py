@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libffnk.so"
 
-OP_LINEAR_FWD, OP_FFN_FWD, OP_LINEAR_BWD, OP_FFN_UP, OP_FFN_DOWN, OP_BWD_DX, OP_BWD_DW = range(7)
+OP_LINEAR_FWD, OP_FFN_FWD, OP_LINEAR_BWD, OP_FFN_UP, OP_FFN_DOWN, OP_BWD_DX, OP_BWD_DW, OP_FFN_BWD = range(8)
 PATH_MFMA_TILED, PATH_STREAM, PATH_GENERIC = range(3)
 
 # Every symbol include/ffnk.h declares, with its ctypes signature.
@@ -34,6 +34,14 @@ _SIGNATURES = {
     "ffnk_masked_linear_bwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64,
                                        c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                        c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "ffnk_masked_ffn_bwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64,            # g, x
+                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,  # W1 W3 U1 U3, strides
+                                    c_void_p, c_void_p, c_int64, c_int64,            # W2 U2, strides
+                                    c_void_p,                                        # mask
+                                    c_void_p, c_int64,                               # dx
+                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,  # dW1 dW3 dU1 dU3
+                                    c_void_p, c_void_p, c_int64, c_int64,            # dW2 dU2
+                                    c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -4,7 +4,7 @@ plain-PyTorch modules (both branches + blend, on the GPU) against the MaskedLine
 modules, and with --check report the L2 distance of outputs (and gradients with --bwd).
 
     python -m ffn_kernel_amd.check linear [--bsz 1] [--bwd] [--check] [--max-mult 4]
-    python -m ffn_kernel_amd.check ffn    [--bsz 1] [--check] [--max-mult 4] [--d 1024] [--h 2048]
+    python -m ffn_kernel_amd.check ffn    [--bsz 1] [--bwd] [--check] [--max-mult 4] [--d 1024] [--h 2048]
 
 Prints one JSON object per sequence length.  Exit status 1 if --check finds a relative L2 distance
 above --tol.
@@ -45,12 +45,15 @@ class TorchFFN(nn.Module):
         self.w1, self.w2, self.w3 = mk(hidden_size, intermediate_size), mk(intermediate_size, hidden_size), mk(hidden_size, intermediate_size)
         self.u1, self.u2, self.u3 = mk(hidden_size, intermediate_size), mk(intermediate_size, hidden_size), mk(hidden_size, intermediate_size)
 
-    @torch.no_grad()
-    def forward(self, x, mask):
+    def blend(self, x, mask):
         m = mask[:, :, None]
         p1 = F.silu(self.w1(x)) * self.w3(x)
         p2 = F.silu(self.u1(x)) * self.u3(x)
         return self.w2(p1) * m + self.u2(p2) * ~m
+
+    @torch.no_grad()
+    def forward(self, x, mask):  # the reference's module is forward-only (test_ffn.py:41)
+        return self.blend(x, mask)
 
 
 def generate_mask(batch_size, seq_len, image_size, rng, device):
@@ -85,7 +88,7 @@ def main(argv=None) -> int:
     ap.add_argument("op", choices=["linear", "ffn"])
     ap.add_argument("--bsz", type=int, default=1)
     ap.add_argument("--check", action="store_true")
-    ap.add_argument("--bwd", action="store_true", help="linear only: include the backward")
+    ap.add_argument("--bwd", action="store_true", help="include the backward")
     ap.add_argument("--max-mult", type=int, default=31, help="sweep seq_len = 2048 * i for i = 1..max-mult")
     ap.add_argument("--d", type=int, default=1024)
     ap.add_argument("--h", type=int, default=2048)
@@ -126,16 +129,28 @@ def main(argv=None) -> int:
                 rec["rel_l2_dx"] = _rel(xs[1].grad, xs[0].grad)
                 rec["rel_l2_dWv"] = _rel(mod.linear_v.weight.grad, ref.linear_v.weight.grad)
                 rec["rel_l2_dWt"] = _rel(mod.linear_t.weight.grad, ref.linear_t.weight.grad)
+            elif args.bwd:
+                xs = []
+                for m, fwd in ((ref, ref.blend), (mod, mod)):
+                    m.zero_grad(set_to_none=True)
+                    xi = x.clone().requires_grad_(True)
+                    o = fwd(xi, mask)
+                    o.sum().backward()
+                    xs.append((xi, o))
+                rec["rel_l2_out"] = _rel(xs[1][1], xs[0][1])
+                rec["rel_l2_dx"] = _rel(xs[1][0].grad, xs[0][0].grad)
+                for k in ("w1", "w2", "w3", "u1", "u2", "u3"):
+                    rec[f"rel_l2_d{k}"] = _rel(getattr(mod, k).weight.grad, getattr(ref, k).weight.grad)
             else:
                 rec["rel_l2_out"] = _rel(mod(x, mask), ref(x, mask))
             rec["ok"] = all(v <= args.tol for k, v in rec.items() if k.startswith("rel_l2"))
             bad |= not rec["ok"]
         else:
             def run(m):
-                if args.op == "linear" and args.bwd:
+                if args.bwd:
                     m.zero_grad(set_to_none=True)
                     xi = x.clone().requires_grad_(True)
-                    m(xi, mask).sum().backward()
+                    (m.blend if isinstance(m, TorchFFN) else m)(xi, mask).sum().backward()
                 else:
                     with torch.no_grad():
                         m(x, mask)

@@ -88,6 +88,34 @@ BwdPlan plan_bwd(int64_t M, int64_t K, int64_t N, bool dw_k_contig) {
   return p;
 }
 
+// MaskedFFN backward workspace: route | T13 [M, 2h] | DH [M, h] | W2^T, U2^T [h, d] | [W1^T|W3^T],
+// [U1^T|U3^T] [d, 2h] | g^T, x^T [d, ldt] | H^T, dt1^T, dt3^T [h, ldt] | fp32 split-K partials.
+struct FfnBwdPlan {
+  BwdPlan up, dn;  // weight-gradient GEMM shapes: up = dW1/dW3 (K = d, N = h), dn = dW2 (K = h, N = d)
+  int64_t ldt;
+  size_t off_t13, off_dh, off_w2t, off_w13t, off_gt, off_xt, off_ht, off_d1t, off_d3t, off_p, total;
+};
+FfnBwdPlan plan_ffn_bwd(int64_t M, int64_t d, int64_t h, bool dup_k_contig, bool ddn_k_contig) {
+  FfnBwdPlan p;
+  p.up = plan_bwd(M, d, h, dup_k_contig);
+  p.dn = plan_bwd(M, h, d, ddn_k_contig);
+  p.ldt = padded_rows(M);
+  const int splits = p.up.tc.splits > p.dn.tc.splits ? p.up.tc.splits : p.dn.tc.splits;
+  size_t o = route_ws_bytes(M);
+  p.off_t13 = o;  o += ws_align((size_t)M * 2 * h * 2);
+  p.off_dh = o;   o += ws_align((size_t)M * h * 2);
+  p.off_w2t = o;  o += 2 * ws_align((size_t)h * d * 2);
+  p.off_w13t = o; o += 2 * ws_align((size_t)d * 2 * h * 2);
+  p.off_gt = o;   o += ws_align((size_t)d * p.ldt * 2);
+  p.off_xt = o;   o += ws_align((size_t)d * p.ldt * 2);
+  p.off_ht = o;   o += ws_align((size_t)h * p.ldt * 2);
+  p.off_d1t = o;  o += ws_align((size_t)h * p.ldt * 2);
+  p.off_d3t = o;  o += ws_align((size_t)h * p.ldt * 2);
+  p.off_p = o;    o += ws_align((size_t)2 * splits * d * h * 4);
+  p.total = o;
+  return p;
+}
+
 // The direct global->LDS path addresses operands with 32-bit byte offsets: from the start of A
 // when its rows are gathered, from the tile's first row otherwise (at most 256 rows away).
 bool direct_ok(int64_t K, int64_t gathered_rows, int64_t lda, int64_t ldb) {
@@ -155,6 +183,14 @@ size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
     case FFNK_OP_LINEAR_BWD: {
       const BwdPlan a = plan_bwd(M, K, N, true), b = plan_bwd(M, K, N, false);
       return a.total > b.total ? a.total : b.total;
+    }
+    case FFNK_OP_FFN_BWD: {
+      size_t best = 0;
+      for (int i = 0; i < 4; ++i) {
+        const size_t t = plan_ffn_bwd(M, K, N, (i & 1) != 0, (i & 2) != 0).total;
+        if (t > best) best = t;
+      }
+      return best;
     }
     default:
       return (size_t)-1;
@@ -444,6 +480,114 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   const int64_t sr = p.dw_k_contig ? dw_stride_n : dw_stride_k;
   const int64_t sc = p.dw_k_contig ? dw_stride_k : dw_stride_n;
   FFNK_HIP(launch_splitk_reduce(P, p.tc.splits, (int)p.R, (int)p.Cc, dWv, dWt, sr, sc, stream), "dW reduce");
+  return FFNK_OK;
+}
+
+int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,
+                        const uint16_t* W1, const uint16_t* W3, const uint16_t* U1, const uint16_t* U3,
+                        int64_t up_stride_k, int64_t up_stride_n, const uint16_t* W2, const uint16_t* U2,
+                        int64_t down_stride_k, int64_t down_stride_n, const uint8_t* mask, uint16_t* dx,
+                        int64_t dx_stride_m, uint16_t* dW1, uint16_t* dW3, uint16_t* dU1, uint16_t* dU3,
+                        int64_t dup_stride_k, int64_t dup_stride_n, uint16_t* dW2, uint16_t* dU2,
+                        int64_t ddown_stride_k, int64_t ddown_stride_n, int64_t M, int64_t d, int64_t h, void* ws,
+                        size_t ws_bytes, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (int e = check_extents(M, d, h)) return e;
+  if (d == 0 || h == 0) return fail(FFNK_E_SHAPE, "MaskedFFN backward needs d > 0 and h > 0");
+  if (!W1 || !W3 || !U1 || !U3 || !W2 || !U2 || !dW1 || !dW3 || !dU1 || !dU3 || !dW2 || !dU2)
+    return fail(FFNK_E_NULL, "weight or weight-gradient pointer is NULL");
+  if (M > 0 && (!g || !x || !mask || !dx)) return fail(FFNK_E_NULL, "g, x, mask or dx is NULL");
+  if (dx_stride_m < d) return fail(FFNK_E_STRIDE, "dx_stride_m=%lld < d=%lld", (long long)dx_stride_m, (long long)d);
+  const bool ok = d % 8 == 0 && h % 8 == 0 && g_stride_m % 8 == 0 && g_stride_m >= d && x_stride_m % 8 == 0 &&
+                  x_stride_m >= d && (M == 0 || (aligned16(g) && aligned16(x))) && up_stride_k == 1 &&
+                  up_stride_n % 8 == 0 && up_stride_n >= d && aligned16(W1) && aligned16(W3) && aligned16(U1) &&
+                  aligned16(U3) && aligned2(W2) && aligned2(U2) && aligned2(dx) && aligned2(dW1) && aligned2(dW3) &&
+                  aligned2(dU1) && aligned2(dU3) && aligned2(dW2) && aligned2(dU2) &&
+                  direct_ok(64, 0, padded_rows(M), padded_rows(M));
+  if (!ok)
+    return fail(FFNK_E_STRIDE, "MaskedFFN backward: d, h and the row strides must be multiples of 8, rows 16-byte "
+                               "aligned and the up-projection weights K-contiguous (up_stride_k == 1)");
+  const FfnBwdPlan p = plan_ffn_bwd(M, d, h, dup_stride_k == 1, ddown_stride_k == 1);
+  if (ws_bytes < p.total || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, p.total);
+  if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
+  uint8_t* wsb = static_cast<uint8_t*>(ws);
+  const RouteWs r = carve_route(wsb, M);
+  uint16_t* T13 = reinterpret_cast<uint16_t*>(wsb + p.off_t13);
+  uint16_t* DH = reinterpret_cast<uint16_t*>(wsb + p.off_dh);
+  const int64_t ld13 = 2 * h;
+  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+
+  // ---- pre-activations, routed order: T13[:, 0:h] = x A1, T13[:, h:2h] = x A3 ----
+  GemmArgs a;
+  a.A = x; a.lda = x_stride_m;
+  a.B1[0] = a.B1[1] = nullptr; a.ldb = up_stride_n;
+  a.ldc = ld13; a.perm = r.perm; a.counts = r.counts;
+  a.M = (int)M; a.N = (int)h; a.K = (int)d;
+  const bool up_direct = direct_ok(d, M, x_stride_m, up_stride_n);
+  a.B0[0] = W1; a.B0[1] = U1; a.C = T13;
+  FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), up_direct, a, stream), "t1 GEMM");
+  a.B0[0] = W3; a.B0[1] = U3; a.C = T13 + h;
+  FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), up_direct, a, stream), "t3 GEMM");
+
+  // ---- dh = gather(g) @ A2^T: contraction over d needs the down weights as [h, d] rows ----
+  const uint16_t* w2t[2] = {W2, U2};
+  int64_t ld2 = down_stride_k;
+  if (!(down_stride_n == 1 && down_stride_k % 8 == 0 && down_stride_k >= d && aligned16(W2) && aligned16(U2))) {
+    uint16_t* c0 = reinterpret_cast<uint16_t*>(wsb + p.off_w2t);
+    uint16_t* c1 = reinterpret_cast<uint16_t*>(wsb + p.off_w2t + ws_align((size_t)h * d * 2));
+    FFNK_HIP(launch_strided_copy2d(W2, down_stride_k, down_stride_n, c0, d, (int)h, (int)d, stream), "weight transpose");
+    FFNK_HIP(launch_strided_copy2d(U2, down_stride_k, down_stride_n, c1, d, (int)h, (int)d, stream), "weight transpose");
+    w2t[0] = c0; w2t[1] = c1; ld2 = d;
+  }
+  a.A = g; a.lda = g_stride_m; a.B0[0] = w2t[0]; a.B0[1] = w2t[1]; a.ldb = ld2;
+  a.C = DH; a.ldc = h;
+  FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), direct_ok(d, M, g_stride_m, ld2), a, stream), "dh GEMM");
+
+  // ---- elementwise: T13 <- (dt1 | dt3), DH <- the SwiGLU intermediate ----
+  FFNK_HIP(launch_swiglu_bwd(T13, ld13, DH, h, (int)M, (int)h, stream), "SwiGLU backward pass");
+
+  // ---- dx = (dt1 | dt3) @ (A1^T | A3^T)^T: one GEMM over the concatenated contraction of length 2h ----
+  uint16_t* w13[2] = {reinterpret_cast<uint16_t*>(wsb + p.off_w13t),
+                      reinterpret_cast<uint16_t*>(wsb + p.off_w13t + ws_align((size_t)d * 2 * h * 2))};
+  FFNK_HIP(launch_strided_copy2d(W1, up_stride_k, up_stride_n, w13[0], ld13, (int)d, (int)h, stream), "weight transpose");
+  FFNK_HIP(launch_strided_copy2d(W3, up_stride_k, up_stride_n, w13[0] + h, ld13, (int)d, (int)h, stream), "weight transpose");
+  FFNK_HIP(launch_strided_copy2d(U1, up_stride_k, up_stride_n, w13[1], ld13, (int)d, (int)h, stream), "weight transpose");
+  FFNK_HIP(launch_strided_copy2d(U3, up_stride_k, up_stride_n, w13[1] + h, ld13, (int)d, (int)h, stream), "weight transpose");
+  GemmArgs b;
+  b.A = T13; b.lda = ld13;
+  b.B0[0] = w13[0]; b.B0[1] = w13[1]; b.B1[0] = b.B1[1] = nullptr; b.ldb = ld13;
+  b.C = dx; b.ldc = dx_stride_m; b.perm = r.perm; b.counts = r.counts;
+  b.M = (int)M; b.N = (int)d; b.K = (int)(2 * h);
+  FFNK_HIP(launch_down_gemm(routed_tile(M, d, false), direct_ok(2 * h, 0, ld13, ld13), b, stream), "dx GEMM");
+
+  // ---- weight gradients: contraction over the rows of each group, on 64-padded transposes ----
+  uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);    // [d, ldt]
+  uint16_t* XT = reinterpret_cast<uint16_t*>(wsb + p.off_xt);    // [d, ldt]
+  uint16_t* HT = reinterpret_cast<uint16_t*>(wsb + p.off_ht);    // [h, ldt]
+  uint16_t* D1T = reinterpret_cast<uint16_t*>(wsb + p.off_d1t);  // [h, ldt]
+  uint16_t* D3T = reinterpret_cast<uint16_t*>(wsb + p.off_d3t);  // [h, ldt]
+  float* P = reinterpret_cast<float*>(wsb + p.off_p);
+  FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, DH, h, (int)h, HT, p.ldt, r.perm, r.counts, (int)M,
+                                    stream, false, true), "g / intermediate transpose");
+  FFNK_HIP(launch_gather_transpose2(x, x_stride_m, (int)d, XT, T13, ld13, (int)h, D1T, p.ldt, r.perm, r.counts,
+                                    (int)M, stream, false, true), "x / dt1 transpose");
+  FFNK_HIP(launch_gather_transpose2(T13 + h, ld13, (int)h, D3T, nullptr, 0, 0, nullptr, p.ldt, r.perm, r.counts,
+                                    (int)M, stream, true, false), "dt3 transpose");
+  auto weight_grad = [&](const BwdPlan& q, const uint16_t* gT, const uint16_t* xT, uint16_t* o0, uint16_t* o1,
+                         int64_t sk, int64_t sn) -> int {
+    SplitKArgs s;
+    s.A = q.dw_k_contig ? gT : xT; s.lda = p.ldt;
+    s.B = q.dw_k_contig ? xT : gT; s.ldb = p.ldt;
+    s.P = P; s.counts = r.counts; s.M = (int)M;
+    s.R = (int)q.R; s.Cc = (int)q.Cc; s.splits = q.tc.splits;
+    FFNK_HIP(launch_splitk_gemm(q.tc.tile, s, stream), "dW split-K GEMM");
+    FFNK_HIP(launch_splitk_reduce(P, q.tc.splits, (int)q.R, (int)q.Cc, o0, o1, q.dw_k_contig ? sn : sk,
+                                  q.dw_k_contig ? sk : sn, stream), "dW reduce");
+    return FFNK_OK;
+  };
+  if (int e = weight_grad(p.dn, GT, HT, dW2, dU2, ddown_stride_k, ddown_stride_n)) return e;
+  if (int e = weight_grad(p.up, D1T, XT, dW1, dU1, dup_stride_k, dup_stride_n)) return e;
+  if (int e = weight_grad(p.up, D3T, XT, dW3, dU3, dup_stride_k, dup_stride_n)) return e;
   return FFNK_OK;
 }
 

@@ -30,6 +30,8 @@ hipError_t launch_linear_gemm(int tile, bool direct, const GemmArgs& g, hipStrea
 hipError_t launch_up_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream);
 // out(token order) = H(routed order) @ W2_g^T
 hipError_t launch_down_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream);
+// C(routed order) = route-gather(A) @ B_g^T (MaskedFFN backward: pre-activations, dH)
+hipError_t launch_gather_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream);
 // P[grp][split] = A[:, kslice] @ B[:, kslice]^T (fp32 partials; weight gradients)
 hipError_t launch_splitk_gemm(int tile, const SplitKArgs& g, hipStream_t stream);
 
@@ -42,7 +44,15 @@ hipError_t launch_strided_copy2d(const uint16_t* src, int64_t sr, int64_t sc, ui
 // [cols, ld_dst]; cols % 8 == 0 and 16-byte aligned source rows are required.
 hipError_t launch_gather_transpose2(const uint16_t* src0, int64_t ld0, int cols0, uint16_t* dst0,
                                     const uint16_t* src1, int64_t ld1, int cols1, uint16_t* dst1, int64_t ld_dst,
-                                    const int32_t* perm, const int32_t* counts, int M, hipStream_t stream);
+                                    const int32_t* perm, const int32_t* counts, int M, hipStream_t stream,
+                                    bool routed0 = false, bool routed1 = false);
+// routedN: source N's rows are already in routed order (row p instead of row perm[p]).
+
+// SwiGLU backward, elementwise and in place over routed-order rows (MaskedFFN backward):
+//   t1 = T13[p, j], t3 = T13[p, h + j], dh = DH[p, j]
+//   T13[p, j] <- dh * t3 * silu'(t1),  T13[p, h + j] <- dh * silu(t1),  DH[p, j] <- silu(t1) * t3
+// T13: [M, 2h] row stride ld13; DH: [M, h] row stride ldh; h % 8 == 0.
+hipError_t launch_swiglu_bwd(uint16_t* T13, int64_t ld13, uint16_t* DH, int64_t ldh, int M, int h, hipStream_t stream);
 // out_g[r * sr + c * sc] = bf16(sum_s P[g][s][r][c]) for g in {0, 1}.
 hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint16_t* out0, uint16_t* out1,
                                 int64_t sr, int64_t sc, hipStream_t stream);

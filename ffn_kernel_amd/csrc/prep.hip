@@ -49,6 +49,7 @@ struct GatherTransposeArgs {
   int cols[2];
   const int32_t* perm; const int32_t* counts;
   int M;
+  int routed[2];  // source rows already in routed order: row p instead of row perm[p]
 };
 
 __global__ __launch_bounds__(256) void gather_transpose_kernel(const GatherTransposeArgs a) {
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(256) void gather_transpose_kernel(const GatherTrans
     uint16_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     const int c = c0 + ch * 8;
     if (valid) {
-      const uint16_t* row = src + (int64_t)a.perm[p] * ld_src;
+      const uint16_t* row = src + (int64_t)(a.routed[z] ? p : a.perm[p]) * ld_src;
       if (c + 8 <= cols) {
         *reinterpret_cast<uint4*>(v) = *reinterpret_cast<const uint4*>(row + c);  // cols % 8 == 0, 16-byte aligned rows
       } else {
@@ -102,16 +103,57 @@ __global__ __launch_bounds__(256) void gather_transpose_kernel(const GatherTrans
 
 hipError_t launch_gather_transpose2(const uint16_t* src0, int64_t ld0, int cols0, uint16_t* dst0,
                                     const uint16_t* src1, int64_t ld1, int cols1, uint16_t* dst1, int64_t ld_dst,
-                                    const int32_t* perm, const int32_t* counts, int M, hipStream_t stream) {
+                                    const int32_t* perm, const int32_t* counts, int M, hipStream_t stream,
+                                    bool routed0, bool routed1) {
   if (M <= 0 || (cols0 <= 0 && cols1 <= 0)) return hipSuccess;
   GatherTransposeArgs a;
   a.src[0] = src0; a.ld_src[0] = ld0; a.dst[0] = dst0; a.cols[0] = cols0;
   a.src[1] = src1; a.ld_src[1] = ld1; a.dst[1] = dst1; a.cols[1] = cols1;
   a.ld_dst = ld_dst; a.perm = perm; a.counts = counts; a.M = M;
+  a.routed[0] = routed0; a.routed[1] = routed1;
   const int max_pos = (int)round_up64(M, 64) + 64;  // >= pad64(nv) + pad64(nt) for every split of M
   const int max_cols = cols0 > cols1 ? cols0 : cols1;
   dim3 grid(cdiv(max_pos, kTt), cdiv(max_cols, kTt), 2);
   hipLaunchKernelGGL(gather_transpose_kernel, grid, dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+// SwiGLU backward in place (see launch.hpp); 8 columns per thread, fp32 maths, bf16 storage.  The
+// derivative is the textbook one, silu'(t) = s + t s (1 - s) with s = sigmoid(t) (the reference's
+// README.md:159-172 sketches this pass; its derivative term there is not this one and is not used).
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(uint16_t* __restrict__ T13, int64_t ld13,
+                                                         uint16_t* __restrict__ DH, int64_t ldh, int M, int h) {
+  const int h8 = h >> 3;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)M * h8) return;
+  const int p = (int)(idx / h8), j = (int)(idx % h8) * 8;
+  uint16_t* pt1 = T13 + (int64_t)p * ld13 + j;
+  uint16_t* pt3 = pt1 + h;
+  uint16_t* pdh = DH + (int64_t)p * ldh + j;
+  uint16_t t1[8], t3[8], dh[8];
+  *reinterpret_cast<uint4*>(t1) = *reinterpret_cast<const uint4*>(pt1);
+  *reinterpret_cast<uint4*>(t3) = *reinterpret_cast<const uint4*>(pt3);
+  *reinterpret_cast<uint4*>(dh) = *reinterpret_cast<const uint4*>(pdh);
+  uint16_t o1[8], o3[8], oh[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float a = bf2f(t1[e]), b = bf2f(t3[e]), g = bf2f(dh[e]);
+    const float s = 1.0f / (1.0f + __expf(-a));
+    const float silu = a * s;
+    o1[e] = f2bf(g * b * (s + silu * (1.0f - s)));
+    o3[e] = f2bf(g * silu);
+    oh[e] = f2bf(silu * b);
+  }
+  *reinterpret_cast<uint4*>(pt1) = *reinterpret_cast<const uint4*>(o1);
+  *reinterpret_cast<uint4*>(pt3) = *reinterpret_cast<const uint4*>(o3);
+  *reinterpret_cast<uint4*>(pdh) = *reinterpret_cast<const uint4*>(oh);
+}
+
+hipError_t launch_swiglu_bwd(uint16_t* T13, int64_t ld13, uint16_t* DH, int64_t ldh, int M, int h, hipStream_t stream) {
+  if (M <= 0 || h <= 0) return hipSuccess;
+  if (h % 8 != 0 || ld13 % 8 != 0 || ldh % 8 != 0) return hipErrorInvalidValue;
+  const int64_t n = (int64_t)M * (h / 8);
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3((unsigned)cdiv64(n, 256)), dim3(256), 0, stream, T13, ld13, DH, ldh, M, h);
   return hipGetLastError();
 }
 

@@ -44,8 +44,10 @@ class MaskedLinearModule(nn.Module):
 
 
 class MaskedFFNModule(nn.Module):
-    """SwiGLU FFN with visual weights (w1, w2, w3) and text weights (u1, u2, u3); forward only,
-    executed under no_grad like the reference's `Triton` module of test_ffn.py."""
+    """SwiGLU FFN with visual weights (w1, w2, w3) and text weights (u1, u2, u3).  The reference's
+    `Triton` module of test_ffn.py / README.md:101-124 runs under no_grad on `.weight.data` because
+    its op has no backward; this one passes the parameters themselves, so it trains as well (wrap the
+    call in torch.no_grad() for inference, as with any module)."""
 
     def __init__(self, hidden_size: int, intermediate_size: int, device=None, dtype=torch.bfloat16):
         super().__init__()
@@ -53,9 +55,8 @@ class MaskedFFNModule(nn.Module):
         self.w1, self.w2, self.w3 = mk(hidden_size, intermediate_size), mk(intermediate_size, hidden_size), mk(hidden_size, intermediate_size)
         self.u1, self.u2, self.u3 = mk(hidden_size, intermediate_size), mk(intermediate_size, hidden_size), mk(hidden_size, intermediate_size)
 
-    @torch.no_grad()
     def forward(self, x: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
         x2, m, batch = _flatten(x, mask)
-        y = MaskedFFN.apply(x2, self.w1.weight.data.T, self.w2.weight.data.T, self.w3.weight.data.T,
-                            self.u1.weight.data.T, self.u2.weight.data.T, self.u3.weight.data.T, m)
+        y = MaskedFFN.apply(x2, self.w1.weight.T, self.w2.weight.T, self.w3.weight.T,
+                            self.u1.weight.T, self.u2.weight.T, self.u3.weight.T, m)
         return _unflatten(y, batch)

@@ -193,6 +193,61 @@ def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask) -> torch.Tensor:
     return out
 
 
+def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask):
+    """(da, dw1, dw2, dw3, du1, du2, du3) of MaskedFFN.  The reference stops at NotImplementedError
+    here (ops.py:34-38); the decomposition follows its README sketch (README.md:159-172): routed
+    GEMMs around one elementwise SwiGLU-gradient pass.  Weight gradients keep the strides of the
+    weight views they belong to, as the linear backward's do."""
+    _require_cuda_bf16("grad", grad, 2)
+    _require_cuda_bf16("a", a, 2)
+    for name, w in (("w1", w1), ("w2", w2), ("w3", w3), ("u1", u1), ("u2", u2), ("u3", u3)):
+        _require_cuda_bf16(name, w, 2)
+    M, d = a.shape
+    h = w1.shape[1]
+    if grad.shape != (M, d):
+        raise ValueError(f"grad shape {tuple(grad.shape)} != {(M, d)}")
+    for name, w in (("w1", w1), ("w3", w3), ("u1", u1), ("u3", u3)):
+        if w.shape != (d, h):
+            raise ValueError(f"{name} shape {tuple(w.shape)} != {(d, h)}")
+    for name, w in (("w2", w2), ("u2", u2)):
+        if w.shape != (h, d):
+            raise ValueError(f"{name} shape {tuple(w.shape)} != {(h, d)}")
+    if d % 8 or h % 8 or d == 0 or h == 0:
+        raise ValueError(f"MaskedFFN backward needs d and h to be positive multiples of 8, got d={d}, h={h}")
+    dev = a.device
+    _same_device(dev, w1=w1, w2=w2, w3=w3, u1=u1, u2=u2, u3=u3, grad=grad)
+    mask = _require_mask(mask, M, dev)
+    grad = _rows_contiguous(grad)
+    a = _rows_contiguous(a)
+    # the up-projection weights must be K-contiguous ([h, d] memory, i.e. nn.Linear.weight.T views)
+    ups = [w if _wstrides(w) == (1, d) else w.t().contiguous().t() for w in (w1, w3, u1, u3)]
+    downs = [_k_major(w) for w in (w2, u2)]
+    if len({_wstrides(w) for w in downs}) != 1:
+        downs = [w.t().contiguous().t() for w in downs]
+    usk, usn = _wstrides(ups[0])
+    dsk, dsn = _wstrides(downs[0])
+    da = torch.empty((M, d), device=dev, dtype=torch.bfloat16)
+    dups = [torch.empty_strided(w1.shape, w1.stride(), device=dev, dtype=torch.bfloat16) for _ in range(4)]
+    ddowns = [torch.empty_strided(w2.shape, w2.stride(), device=dev, dtype=torch.bfloat16) for _ in range(2)]
+    gusk, gusn = _wstrides(dups[0])
+    gdsk, gdsn = _wstrides(ddowns[0])
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
+        ws = _workspace(ws_bytes, dev)
+        rc = lib.ffnk_masked_ffn_bwd(grad.data_ptr(), grad.stride(0) if M > 1 else d, a.data_ptr(),
+                                     a.stride(0) if M > 1 else d, ups[0].data_ptr(), ups[1].data_ptr(),
+                                     ups[2].data_ptr(), ups[3].data_ptr(), usk, usn, downs[0].data_ptr(),
+                                     downs[1].data_ptr(), dsk, dsn, mask.data_ptr(), da.data_ptr(), d,
+                                     dups[0].data_ptr(), dups[1].data_ptr(), dups[2].data_ptr(), dups[3].data_ptr(),
+                                     gusk, gusn, ddowns[0].data_ptr(), ddowns[1].data_ptr(), gdsk, gdsn, M, d, h,
+                                     ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+    _lib.check(rc, "ffnk_masked_ffn_bwd")
+    dw1, dw3, du1, du3 = dups
+    dw2, du2 = ddowns
+    return da, dw1, dw2, dw3, du1, du2, du3
+
+
 class MaskedLinear(Function):
     """c = a @ (b1 where mask else b2), forward and backward (reference: ops.py:9-24)."""
 
@@ -213,15 +268,19 @@ class MaskedLinear(Function):
 
 
 class MaskedFFN(Function):
-    """Routed SwiGLU FFN, forward only like the reference (ops.py:27-38)."""
+    """Routed SwiGLU FFN (reference: ops.py:27-38).  The backward, which the reference leaves at
+    NotImplementedError, recomputes the pre-activations from the saved inputs."""
 
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, a, w1, w2, w3, u1, u2, u3, mask):
+        ctx.save_for_backward(a, mask)
+        ctx.weights = (w1, w2, w3, u1, u2, u3)
         return masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask)
 
     @staticmethod
     @once_differentiable
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad):
-        raise NotImplementedError
+        a, mask = ctx.saved_tensors
+        return (*masked_ffn_backward(grad, a, *ctx.weights, mask), None)

@@ -53,7 +53,8 @@ enum {
   FFNK_OP_FFN_UP = 3,     /* tile_config only: up-projection + SwiGLU stage         */
   FFNK_OP_FFN_DOWN = 4,   /* tile_config only: down-projection stage                */
   FFNK_OP_BWD_DX = 5,     /* tile_config only: dx GEMM of the backward              */
-  FFNK_OP_BWD_DW = 6      /* tile_config only: dW GEMM of the backward              */
+  FFNK_OP_BWD_DW = 6,     /* tile_config only: dW GEMM of the backward              */
+  FFNK_OP_FFN_BWD = 7     /* workspace_bytes only: MaskedFFN backward (K = d, N = h) */
 };
 
 /* kernel families reported by ffnk_tile_config */
@@ -181,6 +182,41 @@ FFNK_API int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m,
                            int64_t dw_stride_k, int64_t dw_stride_n,
                            int64_t M, int64_t K, int64_t N,
                            void* ws, size_t ws_bytes, void* stream);
+
+/*
+ * MaskedFFN backward.  The reference declares it but raises NotImplementedError
+ * (ffn_kernel/ops.py:34-38); its README (README.md:159-172) sketches the decomposition used
+ * here: an elementwise SwiGLU-gradient pass between routed GEMMs.  For row m with
+ * (A1, A2, A3) = mask[m] ? (W1, W2, W3) : (U1, U2, U3), t1 = x[m] @ A1, t3 = x[m] @ A3:
+ *   dh  = g[m] @ A2^T
+ *   dt1 = dh * t3 * silu'(t1),  dt3 = dh * silu(t1),  silu'(t) = s + t s (1 - s), s = sigmoid(t)
+ *   dx[m] = dt1 @ A1^T + dt3 @ A3^T
+ *   dA1 = sum over the group's rows of x[m]^T dt1,  dA3 likewise with dt3,
+ *   dA2 = sum of (silu(t1) * t3)^T g[m]            (exact zeros for an empty group)
+ * g: [M, d]; x: [M, d]; weights and strides as in ffnk_masked_ffn_fwd, with the up-projection
+ * weights K-contiguous (up_stride_k == 1: the nn.Linear.weight.T views the reference passes);
+ * dW1/dW3/dU1/dU3: logical [d, h] with strides (dup_stride_k, dup_stride_n); dW2/dU2: logical
+ * [h, d] with strides (ddown_stride_k, ddown_stride_n).  t1, t3, dh, dt1, dt3 and the
+ * intermediate are held in bf16 between the GEMMs (the forward does the same for the
+ * intermediate); accumulation is fp32; deterministic, no atomics.
+ * Workspace: ffnk_workspace_bytes(FFNK_OP_FFN_BWD, M, d, h).  Layouts outside the above
+ * (d or h not a multiple of 8, unaligned rows, up_stride_k != 1) return FFNK_E_STRIDE.
+ */
+FFNK_API int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m,
+                        const uint16_t* x, int64_t x_stride_m,
+                        const uint16_t* W1, const uint16_t* W3,
+                        const uint16_t* U1, const uint16_t* U3,
+                        int64_t up_stride_k, int64_t up_stride_n,
+                        const uint16_t* W2, const uint16_t* U2,
+                        int64_t down_stride_k, int64_t down_stride_n,
+                        const uint8_t* mask,
+                        uint16_t* dx, int64_t dx_stride_m,
+                        uint16_t* dW1, uint16_t* dW3, uint16_t* dU1, uint16_t* dU3,
+                        int64_t dup_stride_k, int64_t dup_stride_n,
+                        uint16_t* dW2, uint16_t* dU2,
+                        int64_t ddown_stride_k, int64_t ddown_stride_n,
+                        int64_t M, int64_t d, int64_t h,
+                        void* ws, size_t ws_bytes, void* stream);
 
 #ifdef __cplusplus
 }

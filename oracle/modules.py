@@ -118,6 +118,42 @@ def linear_backward_autograd(g, x, Wv, Wt, mask, dtype=torch.float32):
     return x.grad, Wv.grad, Wt.grad
 
 
+def ffn_backward_select(g, x, W, mask, dtype=torch.float64, round_intermediates=False):
+    """Gradients of out = ffn_select(x, W, mask) for upstream gradient g [M, d], by the chain rule
+    written out row-selected (the decomposition README.md:159-172 sketches; silu'(t) is the textbook
+    s + t s (1 - s), not the README's term).  Returns (dx [M, d], dict of weight gradients in
+    nn.Linear layout: w1, w3, u1, u3 [h, d]; w2, u2 [d, h]).  round_intermediates=True rounds
+    t1, t3, dh, dt1, dt3 and the intermediate to bf16 where a kernel that stores them in bf16 does."""
+    rnd = (lambda t: t.to(torch.bfloat16).to(dtype)) if round_intermediates else (lambda t: t)
+    gd, xd = g.to(dtype), x.to(dtype)
+    dx = torch.empty_like(xd)
+    dW = {}
+    for sel, (k1, k2, k3) in ((mask, ("w1", "w2", "w3")), (~mask, ("u1", "u2", "u3"))):
+        xs, gs = xd[sel], gd[sel]
+        A1, A2, A3 = W[k1].to(dtype), W[k2].to(dtype), W[k3].to(dtype)
+        t1, t3 = rnd(xs @ A1.T), rnd(xs @ A3.T)
+        dh = rnd(gs @ A2)
+        s = torch.sigmoid(t1)
+        silu = t1 * s
+        dt1 = rnd(dh * t3 * (s + silu * (1 - s)))
+        dt3 = rnd(dh * silu)
+        hmid = rnd(silu * t3)
+        dx[sel] = dt1 @ A1 + dt3 @ A3
+        dW[k1] = dt1.T @ xs
+        dW[k3] = dt3.T @ xs
+        dW[k2] = gs.T @ hmid
+    return dx, dW
+
+
+def ffn_backward_autograd(g, x, W, mask, dtype=torch.float64):
+    """The same gradients through autograd of the blend form (the reference's oracle module maths)."""
+    xr = x.to(dtype).clone().requires_grad_(True)
+    Wr = {k: v.to(dtype).clone().requires_grad_(True) for k, v in W.items()}
+    out = ffn_blend(xr, Wr, mask)
+    out.backward(g.to(dtype))
+    return xr.grad, {k: v.grad for k, v in Wr.items()}
+
+
 # ----------------------------------------------------------------------------- tolerances
 MAX_ABS_TOL = 2e-2
 REL_L2_TOL = 5e-3

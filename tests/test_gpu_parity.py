@@ -13,7 +13,7 @@ from ffn_kernel_amd import MaskedFFN, MaskedLinear, _lib
 from ffn_kernel_amd import workloads as wl
 from oracle import cref
 from oracle import modules as om
-from helpers import assert_close, assert_close_bf16_pair, note
+from helpers import assert_close, assert_close_bf16_pair, assert_close_pipeline, note
 
 pytestmark = pytest.mark.gpu
 
@@ -309,15 +309,73 @@ def test_ffn_closed_forms(dev):
         assert_close(out[~mask], ref[~mask], "text rows")
 
 
-def test_ffn_backward_raises(dev):
-    note("ffn backward raises")
-    w = wl.make_ffn("t", 8, 64, 64, torch.ones(8, dtype=torch.bool), seed=1).to(dev)
-    x = w.x.clone().requires_grad_(True)
-    args = list(w.op_args())
-    args[0] = x
-    out = MaskedFFN.apply(*args)
-    with pytest.raises(NotImplementedError):
-        out.sum().backward()
+# ------------------------------------------------------------------ MaskedFFN backward
+FFN_BWD_SHAPES = [
+    (37, 64, 128, 0.5),
+    (64, 64, 64, 1.0),      # no text rows: dU* must be exact zeros
+    (64, 64, 64, 0.0),
+    (300, 256, 512, 0.5),
+    (1000, 512, 384, 0.3),
+    (2048, 1024, 2048, 0.5),
+]
+
+
+@pytest.mark.parametrize("M,d,h,p", FFN_BWD_SHAPES)
+def test_ffn_bwd_vs_oracle(dev, M, d, h, p):
+    """The reference raises NotImplementedError here (ops.py:34-38); the oracle is the chain rule of
+    its PyTorch module (pinned on the CPU against autograd and finite differences)."""
+    note(f"ffn bwd M={M} d={d} h={h} p={p}")
+    gen = torch.Generator().manual_seed(M + d + h + 3)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_ffn("t", M, d, h, mask, seed=M + 2, w_std=0.05)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16)
+    dw = w.to(dev)
+    x = dw.x.clone().requires_grad_(True)
+    Wp = {k: v.clone().requires_grad_(True) for k, v in dw.W.items()}
+    out = MaskedFFN.apply(x, Wp["w1"].T, Wp["w2"].T, Wp["w3"].T, Wp["u1"].T, Wp["u2"].T, Wp["u3"].T, dw.mask)
+    out.backward(g.to(dev))
+    torch.cuda.synchronize()
+    # exact chain rule with the intermediates rounded to bf16 where the kernels store them in bf16
+    dx, dW = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64, round_intermediates=True)
+    assert x.grad.shape == (M, d)
+    assert_close_pipeline(x.grad, dx, "dx")
+    for k in ("w1", "w2", "w3", "u1", "u2", "u3"):
+        assert Wp[k].grad.shape == w.W[k].shape and Wp[k].grad.is_contiguous()
+        assert_close_pipeline(Wp[k].grad, dW[k], f"d{k}")
+    # and against the unrounded maths, at bf16-pipeline accuracy
+    dx_e, dW_e = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64)
+    rep = om.error_report(x.grad.float().cpu(), dx_e)
+    assert rep["rel_l2"] <= 1.5e-2, rep
+    for k in dW_e:
+        rep = om.error_report(Wp[k].grad.float().cpu(), dW_e[k])
+        assert rep["rel_l2"] <= 1.5e-2 or dW_e[k].abs().max() == 0, (k, rep)
+    absent = ("u1", "u2", "u3") if p == 1.0 else ("w1", "w2", "w3") if p == 0.0 else ()
+    for k in absent:
+        assert (Wp[k].grad == 0).all()
+
+
+def test_ffn_bwd_is_deterministic_and_validates(dev):
+    note("ffn bwd determinism / validation")
+    from ffn_kernel_amd.ops import masked_ffn_backward
+    mask = torch.rand(500, generator=torch.Generator().manual_seed(5)) < 0.5
+    w = wl.make_ffn("t", 500, 128, 256, mask, seed=9, w_std=0.05).to(dev)
+    g = torch.randn(500, 128, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16).to(dev)
+    args = (g, w.x, w.W["w1"].T, w.W["w2"].T, w.W["w3"].T, w.W["u1"].T, w.W["u2"].T, w.W["u3"].T, w.mask)
+    a = masked_ffn_backward(*args)
+    b = masked_ffn_backward(*args)
+    for ta, tb in zip(a, b):
+        assert torch.equal(ta, tb)
+    # weights given in the other layout ([d, h] memory) are re-laid, gradients keep the caller's strides
+    Wc = {k: v.T.contiguous() for k, v in w.W.items()}
+    c = masked_ffn_backward(g, w.x, Wc["w1"], Wc["w2"], Wc["w3"], Wc["u1"], Wc["u2"], Wc["u3"], w.mask)
+    assert c[1].is_contiguous() and c[1].shape == (128, 256)
+    for ta, tc in zip(a, c):
+        assert_close_bf16_pair(tc, ta.float().cpu(), "layout variant")
+    with pytest.raises(ValueError):
+        masked_ffn_backward(g[:, :100], w.x, *args[2:])
+    bad = wl.make_ffn("t", 8, 60, 64, torch.ones(8, dtype=torch.bool), seed=1).to(dev)
+    with pytest.raises(ValueError):
+        masked_ffn_backward(bad.x, bad.x, *[bad.W[k].T for k in ("w1", "w2", "w3", "u1", "u2", "u3")], bad.mask)
 
 
 # ------------------------------------------------------------------ MaskedLinear backward
@@ -420,3 +478,14 @@ def test_modules_match_reference_modules(dev):
     assert_close_bf16_pair(out, ref_ffn(x, mask).float(), "module ffn vs reference module")
     out2 = ffn(x.to(dev).flatten(0, 1), mask.to(dev).flatten())
     assert torch.equal(out2, out.flatten(0, 1))
+    # the FFN module trains: gradients of its parameters against the exact chain rule
+    g = torch.randn(B, S, D, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    xf = x.to(dev).requires_grad_(True)
+    ffn.zero_grad(set_to_none=True)
+    ffn(xf, mask.to(dev)).backward(g.to(dev))
+    W = {k: getattr(ref_ffn, k).weight.detach() for k in ("w1", "w2", "w3", "u1", "u2", "u3")}
+    dx, dW = om.ffn_backward_select(g.flatten(0, 1), x.flatten(0, 1), W, mask.flatten(), torch.float64,
+                                    round_intermediates=True)
+    assert_close_pipeline(xf.grad.flatten(0, 1), dx, "module ffn dx")
+    for k in W:
+        assert_close_pipeline(getattr(ffn, k).weight.grad, dW[k], f"module ffn d{k}")

@@ -212,6 +212,71 @@ def test_backward_finite_differences():
                 assert abs(fd - grad[i, j]) < 1e-6
 
 
+# ------------------------------------------------------------------ FFN backward
+def _mk_ffn_bwd(M, d, h, p, seed):
+    gen = torch.Generator().manual_seed(seed)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_ffn("t", M, d, h, mask, seed=seed, w_std=0.3)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16)
+    return w, g
+
+
+def test_ffn_backward_select_matches_autograd():
+    for (M, d, h, p) in [(23, 16, 24, 0.5), (9, 8, 8, 0.3), (16, 8, 16, 1.0), (16, 8, 16, 0.0)]:
+        w, g = _mk_ffn_bwd(M, d, h, p, M)
+        dx, dW = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64)
+        dx2, dW2 = om.ffn_backward_autograd(g, w.x, w.W, w.mask, torch.float64)
+        assert torch.allclose(dx, dx2, atol=1e-10, rtol=0)
+        for k in dW:
+            assert torch.allclose(dW[k], dW2[k], atol=1e-10, rtol=0), k
+        absent = ("u1", "u2", "u3") if p == 1.0 else ("w1", "w2", "w3") if p == 0.0 else ()
+        for k in absent:
+            assert (dW[k] == 0).all()
+
+
+def test_ffn_backward_finite_differences():
+    w, g = _mk_ffn_bwd(5, 4, 6, 0.5, 29)
+    w.mask[0], w.mask[1] = True, False  # both groups present
+    x = w.x.double()
+    W = {k: v.double() for k, v in w.W.items()}
+    gd = g.double()
+    f = lambda x_, W_: (om.ffn_select(x_, W_, w.mask, torch.float64) * gd).sum()
+    dx, dW = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64)
+    eps = 1e-6
+    for i in range(x.shape[0]):
+        for j in range(x.shape[1]):
+            xp = x.clone(); xp[i, j] += eps
+            xm = x.clone(); xm[i, j] -= eps
+            assert abs((f(xp, W) - f(xm, W)) / (2 * eps) - dx[i, j]) < 1e-6
+    for k in W:
+        for (i, j) in [(0, 0), (1, 2), (W[k].shape[0] - 1, W[k].shape[1] - 1)]:
+            Wp = dict(W); Wp[k] = W[k].clone(); Wp[k][i, j] += eps
+            Wm = dict(W); Wm[k] = W[k].clone(); Wm[k][i, j] -= eps
+            assert abs((f(x, Wp) - f(x, Wm)) / (2 * eps) - dW[k][i, j]) < 1e-6, k
+
+
+def test_ffn_backward_reductions():
+    # a constant, large gate makes silu the identity and silu' one: the FFN is then the product of
+    # two linear maps through t3, whose gradients are plain matrix products
+    M, d, h = 12, 8, 16
+    w, g = _mk_ffn_bwd(M, d, h, 1.0, 3)
+    x = w.x.double(); x[:, 0] = 1.0
+    W = {k: v.double() for k, v in w.W.items()}
+    W["w1"] = torch.zeros(h, d, dtype=torch.float64); W["w1"][:, 0] = 40.0  # t1 = 40 everywhere
+    dx, dW = om.ffn_backward_select(g, x, W, w.mask, torch.float64)
+    gd = g.double()
+    dh = gd @ W["w2"]
+    assert torch.allclose(dW["w3"], (dh * 40.0).T @ x, atol=1e-8, rtol=1e-12)
+    assert torch.allclose(dW["w2"], gd.T @ (40.0 * (x @ W["w3"].T)), atol=1e-8, rtol=1e-12)
+    # the bf16-rounded variant stays within bf16 accuracy of the exact one
+    w2, g2 = _mk_ffn_bwd(64, 32, 48, 0.5, 5)
+    a = om.ffn_backward_select(g2, w2.x, w2.W, w2.mask, torch.float64)
+    b = om.ffn_backward_select(g2, w2.x, w2.W, w2.mask, torch.float64, round_intermediates=True)
+    assert om.error_report(b[0], a[0])["rel_l2"] < 1e-2
+    for k in a[1]:
+        assert om.error_report(b[1][k], a[1][k])["rel_l2"] < 1e-2
+
+
 # ------------------------------------------------------------------ tolerance helper
 def test_error_report_flags_a_wrong_row():
     w = _mk_linear(64, 32, 32, 0.5, 17)
