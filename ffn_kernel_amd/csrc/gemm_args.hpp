@@ -15,6 +15,12 @@ struct GemmArgs {
   const int32_t* perm;   // routed position -> token row
   const int32_t* counts; // counts[0] = visual rows (device memory)
   int M, N, K;           // N = output columns
+  // Tile schedule.  The order of macro tiles is computed on a grid of sched_bm x sched_bn output
+  // tiles (0 = the kernel's own tile).  tail_mode 0: the launch covers every tile.  1: only the tiles
+  // that fill whole rounds of the chip (the first floor(tiles / 256) * 256 of the order).  2: only the
+  // remaining tiles, each cut into the kernel's own (smaller) tiles - launched with a smaller tile
+  // config, this spreads the last, partial round over all CUs instead of leaving most of them idle.
+  int sched_bm = 0, sched_bn = 0, tail_mode = 0;
 };
 
 // Grouped split-K GEMM used for the weight gradients:

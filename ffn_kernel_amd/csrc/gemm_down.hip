@@ -5,7 +5,7 @@
 namespace ffnk {
 
 hipError_t launch_down_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream) {
-  return direct ? dispatch_tile<PlainTiles<false, true, true>>(tile, g, stream)
+  return direct ? dispatch_tile_with_tail<PlainTiles<false, true, true>>(tile, g, stream)
                 : dispatch_tile<PlainTiles<false, true, false>>(tile, g, stream);
 }
 

@@ -6,7 +6,7 @@
 namespace ffnk {
 
 hipError_t launch_gather_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream) {
-  return direct ? dispatch_tile<PlainTiles<true, false, true>>(tile, g, stream)
+  return direct ? dispatch_tile_with_tail<PlainTiles<true, false, true>>(tile, g, stream)
                 : dispatch_tile<PlainTiles<true, false, false>>(tile, g, stream);
 }
 

@@ -214,13 +214,20 @@ __device__ __forceinline__ void gemm_mainloop_ring(const RingLanes<Cfg>& rl,
   load_frags(0, 0, 0);
 
   auto body = [&](int u, int i, bool full) {
+#ifdef FFNK_X_PRIO
+    __builtin_amdgcn_s_setprio(0);
+#endif
     if (full || i + NS - 2 < nh) ring_wait_barrier<(NS - 3) * L>();
     else ring_wait_barrier<0>();
+#ifdef FFNK_X_PRIO
+    __builtin_amdgcn_s_setprio(FFNK_X_PRIO);
+#endif
     if (full || i + NS - 1 < nh) issue((u + NS - 1) % NS, i + NS - 1);
     load_frags(1, u, 1);
     mfmas(0);
     if (full || i + 1 < nh) load_frags(0, (u + 1) % NS, 0);
     mfmas(1);
+#ifndef FFNK_X_NOSCHED
     if (full) {
       // Issue order inside the (branch-free) steady-state iteration: one LDS read after each of
       // the first TM+TN MFMAs of a K step; the L global->LDS loads spread evenly over the MFMAs
@@ -237,6 +244,7 @@ __device__ __forceinline__ void gemm_mainloop_ring(const RingLanes<Cfg>& rl,
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
     }
+#endif
   };
   int i0 = 0;
   for (; i0 + 2 * NS - 2 < nh; i0 += NS) {  // every guard inside is true: no branches
@@ -362,6 +370,8 @@ __device__ __forceinline__ void gemm_mainloop_staged(const TileLanes<Cfg>& tl,
 // Map a launch-order workgroup id to a position L in the tile order such that every XCD
 // (workgroup b runs on XCD b % 8) owns one contiguous range of the order: tiles that share
 // A rows / B columns then meet in the same L2.  Returns -1 for a surplus workgroup.
+constexpr int kCusPerChip = 256;
+
 __device__ __forceinline__ int xcd_tile_slot(int total) {
   const int per_xcd = cdiv(total, kXcds);
   const int slot = blockIdx.x / kXcds;
@@ -421,12 +431,29 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   __shared__ __attribute__((aligned(1024))) uint8_t lds[Cfg::LDS_BYTES];
 
   // ---- tile schedule (all from device-side counts; no host sync) ----
+  const int SBM = g.sched_bm > 0 ? g.sched_bm : BM;
+  const int SBN = g.sched_bn > 0 ? g.sched_bn : Cfg::BN_OUT;
   const int n_vis = g.counts[0];
   const int n_txt = g.M - n_vis;
-  const int tiles_v = cdiv(n_vis, BM);
-  const int tiles_m = tiles_v + cdiv(n_txt, BM);
-  const int tiles_n = cdiv(g.N, Cfg::BN_OUT);
-  const int L = xcd_tile_slot(tiles_m * tiles_n);
+  const int tiles_v = cdiv(n_vis, SBM);
+  const int tiles_m = tiles_v + cdiv(n_txt, SBM);
+  const int tiles_n = cdiv(g.N, SBN);
+  const int total = tiles_m * tiles_n;
+  int L, sub_m = 0, sub_n = 0;
+  if (g.tail_mode == 0) {
+    L = xcd_tile_slot(total);
+  } else {
+    const int full = total / kCusPerChip * kCusPerChip;
+    if (g.tail_mode == 1) {
+      L = xcd_tile_slot(full);
+    } else {
+      const int qn = SBN / Cfg::BN_OUT, q = (SBM / BM) * qn;  // own tiles per macro tile
+      if ((int)blockIdx.x >= (total - full) * q) return;
+      L = full + (int)blockIdx.x / q;
+      sub_m = ((int)blockIdx.x % q) / qn;
+      sub_n = ((int)blockIdx.x % q) % qn;
+    }
+  }
   if (L < 0) return;
   const int width = Cfg::GROUP_M * tiles_n;
   const int first_m = (L / width) * Cfg::GROUP_M;
@@ -435,9 +462,10 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   const int tile_n = (L % width) / gsz;
 
   const int grp = tile_m < tiles_v ? 0 : 1;
-  const int row0 = grp == 0 ? tile_m * BM : n_vis + (tile_m - tiles_v) * BM;  // routed position
+  const int row0 = (grp == 0 ? tile_m * SBM : n_vis + (tile_m - tiles_v) * SBM) + sub_m * BM;  // routed position
   const int row_end = grp == 0 ? n_vis : g.M;
-  const int n0 = tile_n * Cfg::BN_OUT;
+  const int n0 = tile_n * SBN + sub_n * Cfg::BN_OUT;
+  if (row0 >= row_end || n0 >= g.N) return;  // a sub-tile past the edge of a partial macro tile
 
   f32x16_t acc[TM][TN];
   if (Cfg::DIRECT) {

@@ -36,4 +36,25 @@ inline hipError_t dispatch_tile(int tile, const GemmArgs& g, hipStream_t stream)
   }
 }
 
+// Plain GEMMs on the 256x256 tile: when the tile count is not a multiple of the CU count, the last
+// round would run a few tiles on a few CUs for a full tile time (2064 tiles at M = 32768, N = 4096:
+// 8 rounds + 16 tiles).  Run the whole rounds with the big tile and the remainder as 128x128
+// tiles of the same schedule in a second launch.  Same K order per output element, so the result
+// does not depend on which launch computed it.
+template <class Tiles>
+inline hipError_t dispatch_tile_with_tail(int tile, const GemmArgs& g, hipStream_t stream) {
+  using Big = typename Tiles::T0;
+  using Small = typename Tiles::T2;
+  if (tile != TILE_256x256_W8 || g.M <= 0 || g.N <= 0) return dispatch_tile<Tiles>(tile, g, stream);
+  GemmArgs a = g;
+  a.tail_mode = 1;
+  if (hipError_t e = launch_routed_gemm<Big>(a, stream)) return e;
+  a.tail_mode = 2;
+  a.sched_bm = Big::BM;
+  a.sched_bn = Big::BN_OUT;
+  constexpr int q = (Big::BM / Small::BM) * (Big::BN_OUT / Small::BN_OUT);
+  hipLaunchKernelGGL(routed_gemm_kernel<Small>, dim3((kCusPerChip - 1) * q), dim3(Small::NT), 0, stream, a);
+  return hipGetLastError();
+}
+
 }  // namespace ffnk
