@@ -214,20 +214,13 @@ __device__ __forceinline__ void gemm_mainloop_ring(const RingLanes<Cfg>& rl,
   load_frags(0, 0, 0);
 
   auto body = [&](int u, int i, bool full) {
-#ifdef FFNK_X_PRIO
-    __builtin_amdgcn_s_setprio(0);
-#endif
     if (full || i + NS - 2 < nh) ring_wait_barrier<(NS - 3) * L>();
     else ring_wait_barrier<0>();
-#ifdef FFNK_X_PRIO
-    __builtin_amdgcn_s_setprio(FFNK_X_PRIO);
-#endif
     if (full || i + NS - 1 < nh) issue((u + NS - 1) % NS, i + NS - 1);
     load_frags(1, u, 1);
     mfmas(0);
     if (full || i + 1 < nh) load_frags(0, (u + 1) % NS, 0);
     mfmas(1);
-#ifndef FFNK_X_NOSCHED
     if (full) {
       // Issue order inside the (branch-free) steady-state iteration: one LDS read after each of
       // the first TM+TN MFMAs of a K step; the L global->LDS loads spread evenly over the MFMAs
@@ -244,7 +237,6 @@ __device__ __forceinline__ void gemm_mainloop_ring(const RingLanes<Cfg>& rl,
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
     }
-#endif
   };
   int i0 = 0;
   for (; i0 + 2 * NS - 2 < nh; i0 += NS) {  // every guard inside is true: no branches
