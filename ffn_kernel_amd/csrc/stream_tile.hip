@@ -31,9 +31,11 @@ constexpr int kTK = 128;    // K elements per chunk (16 pieces of 16 bytes per r
 // (sharing one token-row slab; fewer wavefronts = less barrier coupling and more workgroups, but
 // every thread then stages more of the slab) and chunks in flight per wavefront (register budget).
 #ifndef FFNK_TILE_SHAPES
-#define FFNK_TILE_SHAPES {2, 4}, {2, 3}, {4, 3}, {4, 3}
+#define FFNK_TILE_SHAPES {2, 4, 0}, {2, 3, 0}, {2, 3, 1}, {2, 3, 1}
 #endif
-struct TileShapeEntry { int waves, depth; };
+// dma: the token-row slab is filled by direct global -> LDS loads (no staging registers, which is
+// what lets the 3- and 4-m-tile shapes run two-wavefront workgroups) instead of through registers.
+struct TileShapeEntry { int waves, depth, dma; };
 constexpr TileShapeEntry kTileShapes[4] = {FFNK_TILE_SHAPES};
 constexpr int kTMaxM = 64;
 
@@ -42,7 +44,7 @@ struct TileJob {
 };
 
 // xs: [2][NTM * 16 token rows][16 pieces] 16-byte slots; wst: this wavefront's [2 tiles][16 rows][16 pieces].
-template <int NTM, bool DUAL, int kTWaves, int kTD>
+template <int NTM, bool DUAL, int kTWaves, int kTD, bool XDMA>
 __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t, const int* s_perm, u32x4_t* xs,
                                           u32x4_t* wst) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -65,17 +67,35 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
   for (int w = 0; w < 2; ++w) wp[w] += (int64_t)(rbase[w] + lq) * a.ldw + kbase + lrow * 8;  // load u adds 4 u rows
   const int64_t w_step = 4 * a.ldw;
 
-  // Token-row slab: two buffers of [NTM * 16 rows][16 pieces].  Each thread stages piece (tid & 15)
-  // of slab rows p * XR + (tid >> 4); slot = row * 16 + (piece ^ row & 15).
-  constexpr int XR = kTWaves * 4;    // slab rows one pass of the workgroup covers
-  constexpr int XP = NTM * 16 / XR;  // passes
+  // Token-row slab, register path: two buffers of [NTM * 16 rows][16 pieces].  Each thread stages
+  // piece (tid & 15) of slab rows p * XR + (tid >> 4); slot = row * 16 + (piece ^ row & 15).
+  constexpr int XR = kTWaves * 4;                  // slab rows one pass of the workgroup covers
+  constexpr int XP = XDMA ? 1 : NTM * 16 / XR;     // passes (register path only)
   const uint16_t* xp[XP];
+  if (!XDMA) {
 #pragma unroll
-  for (int p = 0; p < XP; ++p) {
-    const int j = p * XR + (tid >> 4);
-    const int pos = t.p0 + min(j, t.mg - 1);  // surplus slab rows repeat the last row; dropped in the epilogue
-    const int64_t src = a.gather_x ? (int64_t)s_perm[pos] : (int64_t)pos;
-    xp[p] = a.X + src * a.ldx + kbase + (tid & 15) * 8;
+    for (int p = 0; p < XP; ++p) {
+      const int j = p * XR + (tid >> 4);
+      const int pos = t.p0 + min(j, t.mg - 1);  // surplus slab rows repeat the last row; dropped in the epilogue
+      const int64_t src = a.gather_x ? (int64_t)s_perm[pos] : (int64_t)pos;
+      xp[p] = a.X + src * a.ldx + kbase + (tid & 15) * 8;
+    }
+  }
+  // Token-row slab, direct path: kTD buffers filled by global -> LDS loads.  One load instruction of a
+  // wavefront fills four consecutive slab rows: lane l writes slot l of that 1 KB, i.e. row
+  // 4 g + (l >> 4), position l & 15, which must hold piece (position ^ row & 15) of the row - the
+  // swizzle is applied on the global side.
+  constexpr int XG = XDMA ? NTM * 4 / kTWaves : 1;  // 4-row groups per wavefront per chunk
+  static_assert(!XDMA || XG * kTWaves == NTM * 4, "slab rows must divide among the wavefronts");
+  uint32_t xoff[XG];
+  if (XDMA) {
+#pragma unroll
+    for (int i = 0; i < XG; ++i) {
+      const int j = 4 * (wave + kTWaves * i) + lq;
+      const int pos = t.p0 + min(j, t.mg - 1);
+      const int64_t src = a.gather_x ? (int64_t)s_perm[pos] : (int64_t)pos;
+      xoff[i] = (uint32_t)((src * a.ldx + kbase + ((lrow ^ (j & 15)) * 8)) * 2);  // bytes; host checks M * ldx < 2^30
+    }
   }
 
   // Workgroups walk their chunk range from different starting chunks (wrapping around): weight rows
@@ -93,7 +113,7 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
       for (int u = 0; u < 4; ++u)
         wr[s][w][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp[w] + u * w_step + ko));
   };
-  u32x4_t xr[kTD][XP];
+  u32x4_t xr[XDMA ? 1 : kTD][XP];
   auto loadx = [&](int s, int c) {
     const int64_t ko = phys(c);
 #pragma unroll
@@ -111,6 +131,43 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes have landed; loads stay in flight
     __builtin_amdgcn_s_barrier();
   };
+  // ---- direct path ----
+#if defined(__HIP_DEVICE_COMPILE__)
+  const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc((void*)a.X, 0, 0xffffffff, 0x00020000);
+#endif
+  auto dma_x = [&](int slot, int c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" ::: "memory");  // the explicit waits below count loads: keep this one where it is written
+    u32x4_t* slab = xs + slot * (NTM * 256);
+    const int ko = phys(c) * 2;
+#pragma unroll
+    for (int i = 0; i < XG; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xrs, (__attribute__((address_space(3))) void*)(slab + (wave + kTWaves * i) * 64),
+                                               16, xoff[i], ko, 0, 0);
+    asm volatile("" ::: "memory");
+#endif
+  };
+  // Loads a wavefront has issued after the slab loads of chunk c + 1 by the end of chunk c's iteration:
+  // weights of c+2 .. c+kTD ... (kTD - 1) x 8, slab loads of c+2 .. c+kTD-1 ... (kTD - 2) x XG.
+  constexpr int kAfterX = (kTD - 1) * 8 + (kTD - 2) * XG;
+  static_assert(kAfterX < 64, "vmcnt is a 6-bit counter");
+  constexpr int kWaitSteady = (kAfterX & 15) | (7 << 4) | ((kAfterX >> 4) << 14);  // vmcnt(kAfterX) lgkmcnt(0)
+  constexpr int kWaitAll = 7 << 4;                                                 // vmcnt(0) lgkmcnt(0)
+  // Make the next chunk's slab visible to the workgroup: own slab loads landed, then barrier.
+  auto slab_barrier = [&](bool steady) {
+    asm volatile("" ::: "memory");
+    if (steady) __builtin_amdgcn_s_waitcnt(kWaitSteady);
+    else __builtin_amdgcn_s_waitcnt(kWaitAll);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  // The slab is read with ds_read_b128 written as inline assembly: a compiler-visible LDS read of an
+  // array that direct loads write makes the compiler drain every load in flight first.  The waits for
+  // these reads are therefore explicit too (slab_wait).
+  const uint32_t xs_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)xs;
+  uint32_t xaddr[4];  // this lane's slab address per k-step: row lrow, piece (4 s + lq) ^ lrow
+#pragma unroll
+  for (int s = 0; s < 4; ++s) xaddr[s] = xs_addr + (uint32_t)(lrow * 16 + ((s * 4 + lq) ^ lrow)) * 16;
 
   f32x4_t acc[2][NTM];
 #pragma unroll
@@ -118,13 +175,17 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
 #pragma unroll
     for (int m = 0; m < NTM; ++m) acc[w][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // One chunk.  STEADY: chunk c + 1 + kTD exists, so every load below is issued unconditionally and
-  // the compiler's load-counter waits are exact; otherwise the loads are guarded, which makes the
-  // compiler wait for more than it needs - only the last 2 kTD chunks of a workgroup run that way.
-  // Loads go out as w(c + kTD), x(c + 1 + kTD): the token rows of a chunk are fetched at the same
-  // distance as its weights, so waiting for them never forces younger weight loads to land.
+  // One chunk.  STEADY: every chunk whose loads this iteration would issue exists, so the loads are
+  // unconditional and the compiler's load-counter waits are exact; otherwise the loads are guarded,
+  // which makes the compiler wait for more than it needs - only the last 2 kTD chunks of a workgroup
+  // run that way.  Register path: loads go out as w(c + kTD), x(c + 1 + kTD).  Direct path: x(c + kTD - 1)
+  // into the slab chunk c - 1 used, then w(c + kTD).  Either way the token rows of a chunk are fetched
+  // right after its weights, so waiting for them never forces younger weight loads to land.
   auto chunk = [&](int u3, int c, auto steady_tag) {
     constexpr bool STEADY = decltype(steady_tag)::value;
+    if (XDMA) {
+      if (STEADY || c + kTD - 1 < nc) dma_x((u3 + kTD - 1) % kTD, c + kTD - 1);
+    }
     // weights of chunk c: registers -> swizzled staging tile
 #pragma unroll
     for (int w = 0; w < 2; ++w)
@@ -134,10 +195,12 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
         wst[w * 256 + row * 16 + (lrow ^ row)] = wr[u3][w][u];
       }
     if (STEADY || c + kTD < nc) loadw(u3, c + kTD);
-    // token rows of chunk c + 1 -> the other slab buffer (its last readers passed the previous barrier)
-    if (STEADY || c + 1 < nc) {
-      stage_x((u3 + 1) % kTD, c + 1);
-      if (STEADY || c + 1 + kTD < nc) loadx((u3 + 1) % kTD, c + 1 + kTD);
+    if (!XDMA) {
+      // token rows of chunk c + 1 -> the other slab buffer (its last readers passed the previous barrier)
+      if (STEADY || c + 1 < nc) {
+        stage_x((u3 + 1) % kTD, c + 1);
+        if (STEADY || c + 1 + kTD < nc) loadx((u3 + 1) % kTD, c + 1 + kTD);
+      }
     }
     const u32x4_t* xb = xs + (c & 1) * (NTM * 256);
 #pragma unroll
@@ -145,27 +208,55 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
       const int piece = (s * 4 + lq) ^ lrow;
       const bf16x8_t wf0 = __builtin_bit_cast(bf16x8_t, wst[lrow * 16 + piece]);
       const bf16x8_t wf1 = __builtin_bit_cast(bf16x8_t, wst[256 + lrow * 16 + piece]);
+      u32x4_t xv[NTM];
+      if (XDMA) {
+#pragma unroll
+        for (int m = 0; m < NTM; ++m)
+          asm volatile("ds_read_b128 %0, %1 offset:%2"
+                       : "=v"(xv[m])
+                       : "v"(xaddr[s]), "n"((u3 * NTM * 256 + m * 256) * 16)
+                       : "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int m = 0; m < NTM; ++m) asm volatile("" : "+v"(xv[m]));  // uses below stay after the wait
+      } else {
+#pragma unroll
+        for (int m = 0; m < NTM; ++m) xv[m] = xb[(m * 16 + lrow) * 16 + piece];
+      }
 #pragma unroll
       for (int m = 0; m < NTM; ++m) {
-        const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, xb[(m * 16 + lrow) * 16 + piece]);
+        const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, xv[m]);
         acc[0][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, xf, acc[0][m], 0, 0, 0);
         acc[1][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, xf, acc[1][m], 0, 0, 0);
       }
     }
-    lds_barrier();  // executed the same number of times by every wavefront (nc is uniform)
+    // the next chunk's slab must be complete, and this chunk's reads done, before anyone moves on
+    // (executed the same number of times by every wavefront: nc is uniform)
+    if (XDMA) slab_barrier(STEADY);
+    else lds_barrier();
   };
 
-  // prologue (nc >= 2 kTD, checked on the host): weights of chunks 0 .. kTD-1, token rows of chunks
-  // 0 .. kTD; chunk 0's go straight to the slab
-  loadx(0, 0);
+  // prologue (nc >= 2 kTD, checked on the host)
+  if (XDMA) {
+    // w(0) x(0) w(1) x(1) ... w(kTD - 1)
 #pragma unroll
-  for (int s = 0; s < kTD; ++s) {
-    loadw(s, s);
-    if (s >= 1) loadx(s, s);
+    for (int s = 0; s < kTD; ++s) {
+      loadw(s, s);
+      if (s < kTD - 1) dma_x(s, s);
+    }
+    slab_barrier(true);
+  } else {
+    // weights of chunks 0 .. kTD-1, token rows of chunks 0 .. kTD; chunk 0's go straight to the slab
+    loadx(0, 0);
+#pragma unroll
+    for (int s = 0; s < kTD; ++s) {
+      loadw(s, s);
+      if (s >= 1) loadx(s, s);
+    }
+    stage_x(0, 0);
+    loadx(0, kTD);
+    lds_barrier();
   }
-  stage_x(0, 0);
-  loadx(0, kTD);
-  lds_barrier();
 
   int c0 = 0;
   for (; c0 + 2 * kTD < nc; c0 += kTD) {
@@ -231,9 +322,9 @@ __device__ __forceinline__ int route64(const uint8_t* mask, int M, int* s_perm, 
 }
 
 // grid.x = 2 groups x splits x row blocks (visual workgroups first); 256 threads.
-template <int NTM_MAX, bool DUAL, int kTWaves, int kTD>
+template <int NTM_MAX, bool DUAL, int kTWaves, int kTD, bool XDMA>
 __global__ __launch_bounds__(kTWaves * kWave, 2) void stream_tile_kernel(const StreamArgs a) {
-  __shared__ u32x4_t xs[2 * NTM_MAX * 256];
+  __shared__ u32x4_t xs[(XDMA ? kTD : 2) * NTM_MAX * 256];
   __shared__ u32x4_t wst_all[kTWaves * 512];
   __shared__ int s_perm[kTMaxM];
   __shared__ int s_nvis;
@@ -255,10 +346,10 @@ __global__ __launch_bounds__(kTWaves * kWave, 2) void stream_tile_kernel(const S
   t.nc = min(t.c0 + cps, n_chunks) - t.c0;
   u32x4_t* wst = wst_all + (threadIdx.x >> 6) * 512;
   const int ntm = cdiv(t.mg, 16);
-  if (NTM_MAX >= 4 && ntm >= 4) tile_rows<(NTM_MAX >= 4 ? 4 : 1), DUAL, kTWaves, kTD>(a, t, s_perm, xs, wst);
-  else if (NTM_MAX >= 3 && ntm == 3) tile_rows<(NTM_MAX >= 3 ? 3 : 1), DUAL, kTWaves, kTD>(a, t, s_perm, xs, wst);
-  else if (NTM_MAX >= 2 && ntm == 2) tile_rows<(NTM_MAX >= 2 ? 2 : 1), DUAL, kTWaves, kTD>(a, t, s_perm, xs, wst);
-  else tile_rows<1, DUAL, kTWaves, kTD>(a, t, s_perm, xs, wst);
+  if (NTM_MAX >= 4 && ntm >= 4) tile_rows<(NTM_MAX >= 4 ? 4 : 1), DUAL, kTWaves, kTD, XDMA>(a, t, s_perm, xs, wst);
+  else if (NTM_MAX >= 3 && ntm == 3) tile_rows<(NTM_MAX >= 3 ? 3 : 1), DUAL, kTWaves, kTD, XDMA>(a, t, s_perm, xs, wst);
+  else if (NTM_MAX >= 2 && ntm == 2) tile_rows<(NTM_MAX >= 2 ? 2 : 1), DUAL, kTWaves, kTD, XDMA>(a, t, s_perm, xs, wst);
+  else tile_rows<1, DUAL, kTWaves, kTD, XDMA>(a, t, s_perm, xs, wst);
 }
 
 static int tile_waves(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].waves; }
@@ -289,8 +380,9 @@ int stream_tile_down_splits(int M, int d, int h) {
 template <int NTM_MAX, bool DUAL>
 static void launch_tile_n(const StreamArgs& a, hipStream_t stream) {
   constexpr int W = kTileShapes[NTM_MAX - 1].waves, D = kTileShapes[NTM_MAX - 1].depth;
+  constexpr bool X = kTileShapes[NTM_MAX - 1].dma != 0;
   const int blocks = 2 * (a.Nrows / ((DUAL ? 16 : 32) * W)) * a.splits;
-  hipLaunchKernelGGL((stream_tile_kernel<NTM_MAX, DUAL, W, D>), dim3(blocks), dim3(W * kWave), 0, stream, a);
+  hipLaunchKernelGGL((stream_tile_kernel<NTM_MAX, DUAL, W, D, X>), dim3(blocks), dim3(W * kWave), 0, stream, a);
 }
 
 template <bool DUAL>
@@ -300,6 +392,7 @@ static hipError_t launch_tile(const StreamArgs& a, hipStream_t stream) {
     return hipErrorInvalidValue;
   const int n_chunks = a.K / kTK;
   if (n_chunks - cdiv(n_chunks, a.splits) * (a.splits - 1) < kTMinChunks) return hipErrorInvalidValue;  // a short split
+  if ((int64_t)a.M * a.ldx >= (1ll << 30)) return hipErrorInvalidValue;  // 32-bit byte offsets into the token rows
   if (DUAL && (a.splits != 1 || a.H == nullptr)) return hipErrorInvalidValue;
   if (!DUAL && a.P == nullptr && (a.splits != 1 || a.out == nullptr)) return hipErrorInvalidValue;
   switch (cdiv(a.M, 16)) {
