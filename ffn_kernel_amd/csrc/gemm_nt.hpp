@@ -159,11 +159,21 @@ __device__ __forceinline__ void gemm_mainloop_ring(const RingLanes<Cfg>& rl,
   constexpr int NM = TM * TN, ND = TM + TN;
   const int wave = rl.wave;
 
+  // The panel bases are uniform over a wavefront (they depend on the wave index only), but where a
+  // base is selected per wave (gate or up weight of the SwiGLU kernels) the compiler cannot see that
+  // and wraps the load in a loop over distinct descriptors: pin those to scalar registers.
+  auto wave_uniform = [](const uint16_t* p) {
+    if (!Cfg::DUAL) return reinterpret_cast<void*>(const_cast<uint16_t*>(p));
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+  };
   __amdgpu_buffer_rsrc_t rsA[NJA], rsB[NJB];
 #pragma unroll
-  for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc((void*)baseA[j], 0, 0xffffffff, 0x00020000);
+  for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseA[j]), 0, 0xffffffff, 0x00020000);
 #pragma unroll
-  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc((void*)baseB[j], 0, 0xffffffff, 0x00020000);
+  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
 
   uint32_t koff[2];
 #pragma unroll
