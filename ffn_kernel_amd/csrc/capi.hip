@@ -373,6 +373,9 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
     u.Nrows = (int)h; u.K = (int)d; u.splits = 1; u.H = H; u.ldh = ldh; u.P = nullptr; u.out = nullptr; u.ldo = 0;
     const bool dot = use_dot_path(M, d, h);
     const bool tiled = use_tile_path(M, d, h);
+    if (tiled && M * x_stride_m >= ((int64_t)1 << 30))
+      return fail(FFNK_E_STRIDE, "x_stride_m=%lld: the decode kernels address the token rows with 32-bit offsets",
+                  (long long)x_stride_m);
     FFNK_HIP(dot ? launch_stream_dot_up(u, stream) : tiled ? launch_stream_tile_up(u, stream) : launch_stream_up(u, stream),
              "streaming up-projection");
     FFNK_HIP(mark(1), "event record");
