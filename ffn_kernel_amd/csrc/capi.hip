@@ -250,6 +250,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
       out->block_n = stream_tile_rows_per_block((int)M, up);
       out->block_k = 128;
       out->lds_stages = stream_tile_depth((int)M);
+      out->direct_lds = stream_tile_direct((int)M);
       out->split_k = up ? 1 : down_splits(M, K, N);
     }
     if (use_dot_path(M, K, N)) {

@@ -355,6 +355,7 @@ __global__ __launch_bounds__(kTWaves * kWave, 2) void stream_tile_kernel(const S
 static int tile_waves(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].waves; }
 
 int stream_tile_rows_per_block(int M, bool dual) { return (dual ? 16 : 32) * tile_waves(M); }
+int stream_tile_direct(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].dma; }
 int stream_tile_depth(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].depth; }
 
 constexpr int kTMinChunks = 8;  // >= 2 x the deepest ring: lets the kernels run an unconditional prologue

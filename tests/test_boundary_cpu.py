@@ -50,9 +50,10 @@ def test_tile_table_entries():
     # 9 <= M <= 64: LDS-transposed streams, 128-element chunks, three in flight, split-K down projection
     mid = _lib.tile_config(_lib.OP_FFN_UP, 64, 4096, 14336)
     assert mid["path"] == _lib.PATH_STREAM and mid["block_k"] == 128 and mid["lds_stages"] == 3
-    assert mid["block_n"] == 64 and mid["split_k"] == 1
+    assert mid["block_n"] == 32 and mid["split_k"] == 1 and mid["direct_lds"] == 1  # two wavefronts, direct slab loads
     assert _lib.tile_config(_lib.OP_FFN_DOWN, 64, 4096, 14336)["split_k"] >= 4
-    assert _lib.tile_config(_lib.OP_FFN_UP, 16, 4096, 14336)["block_n"] == 32  # two wavefronts per workgroup
+    low = _lib.tile_config(_lib.OP_FFN_UP, 16, 4096, 14336)
+    assert low["block_n"] == 32 and low["direct_lds"] == 0 and low["lds_stages"] == 4  # slab through registers
     # small M whose extents are not whole 512-element slices run on the LDS-transposed streams too ...
     odd = _lib.tile_config(_lib.OP_FFN_UP, 4, 1152, 1408)
     assert odd["path"] == _lib.PATH_STREAM and odd["lds_stages"] >= 3
