@@ -9,10 +9,17 @@
 //   * each chunk is transposed through a wave-private, XOR-swizzled LDS tile (ds_write_b128 in load
 //     layout, ds_read_b128 in MFMA fragment layout, both bank-conflict free; one wavefront's LDS
 //     operations execute in order, so the tile needs neither double buffering nor waits);
-//   * the token rows of the chunk (x, or the SwiGLU intermediate) are staged once per workgroup in a
-//     double-buffered LDS slab that the wavefronts of the workgroup share, fetched at the same distance as the
-//     weights so that the in-order load counter never forces a weight load to complete early;
-//   * one raw s_barrier per chunk hands the slab over; it does not drain the loads in flight.
+//   * the token rows of the chunk (x, or the SwiGLU intermediate) are staged once per workgroup in an
+//     LDS slab that its wavefronts share.  For up to two m-tiles the slab is double-buffered and goes
+//     through registers, fetched at the same distance as the weights so that the in-order load
+//     counter never forces a weight load to complete early.  For three and four m-tiles the staging
+//     registers would not fit beside the weight ring, so the slab is a ring of buffers filled by
+//     direct global -> LDS loads (swizzled on the global side) and read with ds_read_b128 written
+//     as inline assembly: a compiler-visible LDS read of an array that direct loads write makes the
+//     compiler drain every load in flight first;
+//   * one raw s_barrier per chunk hands the slab over; it does not drain the loads in flight;
+//   * the K loop is split into a branch-free steady part and a guarded tail: a load behind a uniform
+//     branch makes the compiler's load-counter waits conservative for the whole loop.
 // The up projection covers all of K in one workgroup (SwiGLU epilogue, routed-order H); the down
 // projection splits K across workgroups into fp32 partials that stream_reduce_kernel sums.
 // Same role as the reference's small-M launches of its GEMM tiles (ffn_kernel/ffn.py:527-560,
