@@ -480,10 +480,12 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   s.B = p.dw_k_contig ? XT : GT; s.ldb = p.ldt;
   s.P = P; s.counts = r.counts; s.M = (int)M;
   s.R = (int)p.R; s.Cc = (int)p.Cc; s.splits = p.tc.splits;
-  FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
   const int64_t sr = p.dw_k_contig ? dw_stride_n : dw_stride_k;
   const int64_t sc = p.dw_k_contig ? dw_stride_k : dw_stride_n;
-  FFNK_HIP(launch_splitk_reduce(P, p.tc.splits, (int)p.R, (int)p.Cc, dWv, dWt, sr, sc, stream), "dW reduce");
+  if (p.tc.splits == 1) { s.out[0] = dWv; s.out[1] = dWt; s.out_sr = sr; s.out_sc = sc; }
+  FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
+  if (p.tc.splits > 1)
+    FFNK_HIP(launch_splitk_reduce(P, p.tc.splits, (int)p.R, (int)p.Cc, dWv, dWt, sr, sc, stream), "dW reduce");
   return FFNK_OK;
 }
 
@@ -584,9 +586,11 @@ int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x
     s.B = q.dw_k_contig ? xT : gT; s.ldb = p.ldt;
     s.P = P; s.counts = r.counts; s.M = (int)M;
     s.R = (int)q.R; s.Cc = (int)q.Cc; s.splits = q.tc.splits;
+    const int64_t sr = q.dw_k_contig ? sn : sk, sc = q.dw_k_contig ? sk : sn;
+    if (q.tc.splits == 1) { s.out[0] = o0; s.out[1] = o1; s.out_sr = sr; s.out_sc = sc; }
     FFNK_HIP(launch_splitk_gemm(q.tc.tile, s, stream), "dW split-K GEMM");
-    FFNK_HIP(launch_splitk_reduce(P, q.tc.splits, (int)q.R, (int)q.Cc, o0, o1, q.dw_k_contig ? sn : sk,
-                                  q.dw_k_contig ? sk : sn, stream), "dW reduce");
+    if (q.tc.splits > 1)
+      FFNK_HIP(launch_splitk_reduce(P, q.tc.splits, (int)q.R, (int)q.Cc, o0, o1, sr, sc, stream), "dW reduce");
     return FFNK_OK;
   };
   if (int e = weight_grad(p.dn, GT, HT, dW2, dU2, ddown_stride_k, ddown_stride_n)) return e;

@@ -35,6 +35,10 @@ struct SplitKArgs {
   const int32_t* counts;
   int M;                           // routed rows in total (both groups)
   int R, Cc, splits;
+  // splits == 1 only: store bf16 results straight to out[grp][r * out_sr + c * out_sc] instead of
+  // fp32 partials (no reduce pass).  NULL: partials go to P.
+  uint16_t* out[2] = {nullptr, nullptr};
+  int64_t out_sr = 0, out_sc = 0;
 };
 
 }  // namespace ffnk

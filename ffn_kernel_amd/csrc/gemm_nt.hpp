@@ -590,6 +590,34 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
 
   // acc[i][j][v]: BM-panel row (= output column c) c0 + wm*WTM + i*32 + (lane&31);
   //               BN-panel row (= output row r) r0 + wn*WTN + j*32 + 8*(v/4) + 4*(lane>>5) + v%4.
+  if (g.out[0] != nullptr) {
+    // single split: the sums are complete, store bf16 with the caller's strides
+    uint16_t* out = g.out[grp];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int c = c0 + rl.wm * Cfg::WTM + i * 32 + (int)rl.lr;
+      if (c >= g.Cc) continue;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int r = r0 + rl.wn * Cfg::WTN_OUT + j * 32 + 8 * q4 + 4 * (int)rl.lh;
+          uint16_t* dst = out + (int64_t)r * g.out_sr + (int64_t)c * g.out_sc;
+          if (g.out_sr == 1 && r + 3 < g.R && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+            uint2 v2;
+            v2.x = pack2bf(acc[i][j][4 * q4], acc[i][j][4 * q4 + 1]);
+            v2.y = pack2bf(acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]);
+            *reinterpret_cast<uint2*>(dst) = v2;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (r + e < g.R) dst[(int64_t)e * g.out_sr] = f2bf(acc[i][j][4 * q4 + e]);  // out_sc == 1: 32 lanes -> 64 contiguous bytes
+          }
+        }
+      }
+    }
+    return;
+  }
   float* P = g.P + ((int64_t)(grp * g.splits + split)) * g.R * g.Cc;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {

@@ -30,9 +30,43 @@ __global__ __launch_bounds__(256) void strided_copy2d_kernel(const uint16_t* __r
   }
 }
 
+// dst[r, c] = src[c * sc + r] (a transpose: the source is contiguous along r).  64x64 tile per block:
+// 16-byte reads along r, scalar transposing LDS writes, 16-byte reads of the transposed tile, 16-byte
+// stores along c.  rows, cols, sc, ld_dst multiples of 8; 16-byte aligned bases.
+__global__ __launch_bounds__(256) void transpose_copy_kernel(const uint16_t* __restrict__ src, int64_t sc,
+                                                             uint16_t* __restrict__ dst, int64_t ld_dst, int rows,
+                                                             int cols) {
+  __shared__ __attribute__((aligned(16))) uint16_t tile[kTt][kTt + 8];  // [r][c]
+  const int r0 = blockIdx.y * kTt, c0 = blockIdx.x * kTt;
+  const int t = threadIdx.x, ch = t & 7;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int ci = (t >> 3) + pass * 32;
+    uint16_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (c0 + ci < cols && r0 + ch * 8 < rows)
+      *reinterpret_cast<uint4*>(v) = *reinterpret_cast<const uint4*>(src + (int64_t)(c0 + ci) * sc + r0 + ch * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) tile[ch * 8 + e][ci] = v[e];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int rr = (t >> 3) + pass * 32;
+    if (r0 + rr < rows && c0 + ch * 8 < cols)
+      *reinterpret_cast<uint4*>(dst + (int64_t)(r0 + rr) * ld_dst + c0 + ch * 8) =
+          *reinterpret_cast<const uint4*>(&tile[rr][ch * 8]);
+  }
+}
+
 hipError_t launch_strided_copy2d(const uint16_t* src, int64_t sr, int64_t sc, uint16_t* dst, int64_t ld_dst,
                                  int rows, int cols, hipStream_t stream) {
   if (rows <= 0 || cols <= 0) return hipSuccess;
+  if (sr == 1 && sc % 8 == 0 && ld_dst % 8 == 0 && rows % 8 == 0 && cols % 8 == 0 &&
+      (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+    dim3 grid(cdiv(cols, kTt), cdiv(rows, kTt));
+    hipLaunchKernelGGL(transpose_copy_kernel, grid, dim3(256), 0, stream, src, sc, dst, ld_dst, rows, cols);
+    return hipGetLastError();
+  }
   dim3 grid(cdiv(cols, kTt), cdiv(rows, kTt));
   hipLaunchKernelGGL(strided_copy2d_kernel, grid, dim3(256), 0, stream, src, sr, sc, dst, ld_dst, rows, cols);
   return hipGetLastError();

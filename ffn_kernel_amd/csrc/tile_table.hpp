@@ -35,6 +35,13 @@ inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual) {
 // Weight-gradient GEMM: two [R, Cc] outputs, contraction over about M / 2 rows each.
 inline TileChoice pick_splitk_tile(int64_t M, int64_t R, int64_t Cc) {
   TileChoice c;
+  // Large outputs: the 256x256 tile fills the chip on its own, no split needed (and the GEMM then
+  // stores bf16 directly, without partials or a reduce pass).
+  if (2 * cdiv64(R, 256) * cdiv64(Cc, 256) >= 2 * kCus) {
+    c.tile = TILE_256x256_W8;
+    c.splits = 1;
+    return c;
+  }
   c.tile = TILE_128x128_W4;
   const int64_t tiles = 2 * cdiv64(R, 128) * cdiv64(Cc, 128);
   int64_t s = cdiv64(2 * kCus, tiles);            // aim at two workgroups per CU
