@@ -29,12 +29,12 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # profiles/ (routed_gemm_kernel_ffn_fwd_M32768_d4096_h14336.txt, stream_*_kernel_ffn_decode_*.txt).
 # Recorded, not measured live: counters cannot be read from inside the process.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg4": (8.3811e6 * 2.0 + 9.2594e5) * 1024,                                   # up-projection kernel
+    "cfg4": (9.4782e6 * 2.0 + 9.3048e5) * 1024,                                   # up-projection kernel
     # decode: all launches of one call (up-projection, down-projection, reduce where there is one)
     "decode1v": (1.1476e5 * 2.0 + 40 + 5.7481e4 * 2.0 + 8) * 1024,
     "decode8": (2.2979e5 * 2.0 + 320 + 1.1568e5 * 2.0 + 64) * 1024,
-    "decode32": (2.3053e5 * 2.0 + 896 + 1.184e5 * 2.0 + 2048 + 1039 * 2.0 + 256) * 1024,
-    "decode64": (2.3159e5 * 2.0 + 1792 + 1.2202e5 * 2.0 + 8193 + 4111 * 2.0 + 512) * 1024,
+    "decode32": (2.3053e5 * 2.0 + 897 + 1.184e5 * 2.0 + 2048 + 1039 * 2.0 + 256) * 1024,
+    "decode64": (2.3159e5 * 2.0 + 1792 + 1.2203e5 * 2.0 + 4096 + 2063 * 2.0 + 512) * 1024,
 }
 
 
