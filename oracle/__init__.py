@@ -19,6 +19,10 @@ How each function is pinned (tests/test_oracle*.py):
   SwiGLU / FFN       silu closed forms (0, large +/-), W3 = 0 or W1 = 0 -> 0, the C loops vs torch
   linear backward    autograd of the blend form, dW_v + dW_t == x^T g, empty modality -> exact
                      zeros, W_v == W_t -> dx == g W^T, fp64 finite differences
+  FFN backward       (the op the reference leaves at NotImplementedError, ops.py:34-38) chain rule
+                     written out vs autograd of the blend form vs the C loops, fp64 finite
+                     differences on x and on entries of all six weights, constant-gate reduction
+                     to plain matrix products, empty modality -> exact zeros
 The reference itself ships no golden vectors, asserts or tolerances for this path
 (test_linear.py:92-124 and test_ffn.py:111-115 only print); the bf16 tolerances used here are
 max-abs <= 2e-2 and rel-L2 <= 5e-3 against an fp32-accumulated result.

@@ -21,8 +21,10 @@ def _load():
         _lib.ref_masked_linear_fwd.argtypes = [c_void_p] * 5 + [c_int64] * 3
         _lib.ref_masked_ffn_fwd.argtypes = [c_void_p] * 9 + [c_int64] * 3 + [c_int]
         _lib.ref_masked_linear_bwd.argtypes = [c_void_p] * 8 + [c_int64] * 3
+        _lib.ref_masked_ffn_bwd.argtypes = [c_void_p] * 16 + [c_int64] * 3 + [c_int]
         _lib.ref_route.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
-        for f in (_lib.ref_masked_linear_fwd, _lib.ref_masked_ffn_fwd, _lib.ref_masked_linear_bwd, _lib.ref_route):
+        for f in (_lib.ref_masked_linear_fwd, _lib.ref_masked_ffn_fwd, _lib.ref_masked_linear_bwd,
+                  _lib.ref_masked_ffn_bwd, _lib.ref_route):
             f.restype = None
     return _lib
 
@@ -66,6 +68,19 @@ def linear_bwd(g, x, Wv, Wt, mask):
     dx = np.zeros((M, K)); dWv = np.zeros((N, K)); dWt = np.zeros((N, K))
     _load().ref_masked_linear_bwd(*[_p(a) for a in arrs], _p(dx), _p(dWv), _p(dWt), M, K, N)
     return torch.from_numpy(dx), torch.from_numpy(dWv), torch.from_numpy(dWt)
+
+
+def ffn_bwd(g, x, W, mask, round_mid: bool = False):
+    """(dx [M, d], dict of weight gradients in nn.Linear layout) from the C loops."""
+    M, d = x.shape
+    h = W["w1"].shape[0]
+    arrs = [_bits(g), _bits(x)] + [_bits(W[k]) for k in ("w1", "w2", "w3", "u1", "u2", "u3")] + [_mask(mask)]
+    dx = np.zeros((M, d))
+    outs = {"w1": np.zeros((h, d)), "w2": np.zeros((d, h)), "w3": np.zeros((h, d)),
+            "u1": np.zeros((h, d)), "u2": np.zeros((d, h)), "u3": np.zeros((h, d))}
+    _load().ref_masked_ffn_bwd(*[_p(a) for a in arrs], _p(dx), *[_p(outs[k]) for k in ("w1", "w2", "w3", "u1", "u2", "u3")],
+                               M, d, h, int(round_mid))
+    return torch.from_numpy(dx), {k: torch.from_numpy(v) for k, v in outs.items()}
 
 
 def route(mask):

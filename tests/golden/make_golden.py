@@ -52,6 +52,14 @@ def main() -> None:
     out_r = cref.ffn_fwd(f.x, f.W, f.mask, round_mid=True)
     np.savez_compressed(HERE / "ffn_decode_M5_d128_h128.npz", x=bits(f.x), mask=f.mask.numpy(),
                         out_round_mid=out_r.numpy(), **{k: bits(v) for k, v in f.W.items()})
+    # MaskedFFN backward (exact chain rule; the op the reference leaves unimplemented)
+    M, d, h = 21, 32, 48
+    mask = torch.rand(M, generator=gen) < 0.5
+    f = wl.make_ffn("golden_ffn_bwd", M, d, h, mask, seed=14, w_std=0.1)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16)
+    dx, dW = cref.ffn_bwd(g, f.x, f.W, f.mask)
+    np.savez_compressed(HERE / "ffn_bwd_M21_d32_h48.npz", x=bits(f.x), g=bits(g), mask=f.mask.numpy(), dx=dx.numpy(),
+                        **{k: bits(v) for k, v in f.W.items()}, **{"d" + k: v.numpy() for k, v in dW.items()})
     print("wrote", sorted(p.name for p in HERE.glob("*.npz")))
 
 

@@ -82,6 +82,23 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.ffnk_masked_linear_fwd(None, 8, None, None, 1, 8, None, None, 8, 0, 8, 8, None, 0, None) == 0
 
 
+def test_ffn_backward_entry_rejects_bad_arguments_without_a_gpu():
+    lib = _lib.load()
+    P = ctypes.c_void_p
+    one = P(16)  # a non-NULL, 16-byte aligned stand-in; rejected calls touch no memory
+    def call(d=64, h=64, up_sk=1, ws=None, ws_bytes=0, dx_stride=64, M=8, g=one):
+        return lib.ffnk_masked_ffn_bwd(g, d, one, d, one, one, one, one, up_sk, d, one, one, 1, h, one, one, dx_stride,
+                                       one, one, one, one, 1, d, one, one, 1, h, M, d, h, ws, ws_bytes, None)
+    assert call(g=None) == -1                       # NULL g
+    assert call(dx_stride=8) == -3                  # dx rows shorter than d
+    assert call(d=60) == -3 and b"multiples of 8" in lib.ffnk_last_error()
+    assert call(up_sk=64) == -3                     # up-projection weights not K-contiguous
+    assert call() == -5                             # no workspace
+    need = _lib.workspace_bytes(_lib.OP_FFN_BWD, 8192, 1024, 2048)
+    assert need >= 8192 * 3 * 2048 * 2              # t1|t3 and dh in bf16, routed order
+    assert need >= _lib.workspace_bytes(_lib.OP_FFN_FWD, 8192, 1024, 2048)
+
+
 def test_ops_validate_inputs():
     x = torch.zeros(4, 8, dtype=torch.bfloat16)
     w = torch.zeros(8, 8, dtype=torch.bfloat16)

@@ -221,14 +221,22 @@ def _mk_ffn_bwd(M, d, h, p, seed):
     return w, g
 
 
-def test_ffn_backward_select_matches_autograd():
+def test_ffn_backward_select_matches_autograd_and_c_loops():
     for (M, d, h, p) in [(23, 16, 24, 0.5), (9, 8, 8, 0.3), (16, 8, 16, 1.0), (16, 8, 16, 0.0)]:
         w, g = _mk_ffn_bwd(M, d, h, p, M)
         dx, dW = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64)
         dx2, dW2 = om.ffn_backward_autograd(g, w.x, w.W, w.mask, torch.float64)
+        dx3, dW3 = cref.ffn_bwd(g, w.x, w.W, w.mask)
         assert torch.allclose(dx, dx2, atol=1e-10, rtol=0)
+        assert torch.allclose(dx, dx3, atol=1e-10, rtol=0)
         for k in dW:
             assert torch.allclose(dW[k], dW2[k], atol=1e-10, rtol=0), k
+            assert torch.allclose(dW[k], dW3[k], atol=1e-10, rtol=0), k
+        # the bf16-storage variant of the C loops rounds where the torch one does
+        dx4, dW4 = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64, round_intermediates=True)
+        dx5, dW5 = cref.ffn_bwd(g, w.x, w.W, w.mask, round_mid=True)
+        assert torch.allclose(dx4, dx5, atol=1e-2, rtol=1e-2)  # a rounding boundary may fall either way
+        assert (dx4 - dx5).abs().median() < 1e-9
         absent = ("u1", "u2", "u3") if p == 1.0 else ("w1", "w2", "w3") if p == 0.0 else ()
         for k in absent:
             assert (dW[k] == 0).all()
