@@ -120,7 +120,7 @@ FfnBwdPlan plan_ffn_bwd(int64_t M, int64_t d, int64_t h, bool dup_k_contig, bool
 // when its rows are gathered, from the tile's first row otherwise (at most 256 rows away).
 bool direct_ok(int64_t K, int64_t gathered_rows, int64_t lda, int64_t ldb) {
   constexpr int64_t k4g = (int64_t)1 << 32;
-  if (K <= 0 || K % 32 != 0) return false;
+  if (K <= 0 || K % 64 != 0) return false;
   if (gathered_rows > 0 && gathered_rows * lda * 2 >= k4g) return false;
   return 256 * lda * 2 < k4g && 256 * ldb * 2 < k4g;
 }
@@ -229,9 +229,9 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->lds_stages = 2;
   out->group_m = 8;
   out->split_k = splits;
-  out->direct_lds = (contraction > 0 && contraction % 32 == 0) ? 1 : 0;
-  out->block_k = out->direct_lds ? 32 : 64;
-  out->lds_stages = out->direct_lds ? 4 : 2;
+  out->direct_lds = (contraction > 0 && contraction % 64 == 0) ? 1 : 0;
+  out->block_k = 64;
+  out->lds_stages = 2;
   if (stream) {
     // Streaming kernels: a workgroup is 16 * RT weight rows x one K range whose four wavefronts
     // take a quarter each; operands go global -> registers, no LDS staging.

@@ -5,10 +5,10 @@
 // (ffn_kernel/linear.py:127-153, ffn_kernel/ffn.py:68-105), which pay two dots and a select
 // on every mixed tile.
 //
-// Data path per workgroup: 64-column K slabs of the A and B panels go global -> LDS (directly,
-// bypassing registers, through a 4-stage ring of 32-column half-slabs; or staged through
-// registers in 64-column slabs when K is not a multiple of 32); wavefronts read 16-byte MFMA
-// fragments from an XOR-swizzled LDS layout and issue v_mfma_f32_32x32x16_bf16.
+// Data path per workgroup: 64-column K slabs of the A and B panels go global -> LDS, two stages
+// deep (directly, bypassing registers, when K is a multiple of 64; staged through registers
+// otherwise); wavefronts read 16-byte MFMA fragments from an XOR-swizzled LDS layout and issue
+// v_mfma_f32_32x32x16_bf16.
 #pragma once
 #include "common.hpp"
 #include "gemm_args.hpp"
@@ -20,27 +20,17 @@ constexpr int kRowBytes = 128;   // kBK * sizeof(bf16)
 constexpr int kXcds = 8;         // MI355X: 8 XCDs, workgroups are dealt to them round-robin
 
 // ---------------------------------------------------------------------------------------------
-// LDS layouts.  Both keep every ds_read_b128 of an MFMA fragment (16 consecutive tile rows, same
-// logical 16-byte chunk, per 16-lane phase) on 16 distinct 16-byte bank groups, and let a
-// wavefront fill LDS in lane order (lane -> 16 bytes at lane * 16), which is what a
-// global->LDS load requires.
-//
-//  * "slab" layout, 128-byte rows (64 K elements): used by the register-staged path.
-//  * "half-slab" layout, 64-byte rows (32 K elements): used by the direct global->LDS ring.
+// LDS layout: a slab holds 128-byte rows (64 K elements).  The swizzle keeps every ds_read_b128 of
+// an MFMA fragment (16 consecutive tile rows, same logical 16-byte chunk, per 16-lane phase) on 16
+// distinct 16-byte bank groups, and lets a wavefront fill LDS in lane order (lane -> 16 bytes at
+// lane * 16), which is what a global->LDS load requires.
 // ---------------------------------------------------------------------------------------------
 __host__ __device__ constexpr uint32_t lds_swizzle(uint32_t r, uint32_t c) {  // c in 0..7
   return ((r >> 1) << 8) | (((((r & 1u) ^ ((r >> 3) & 1u)) << 3) | (c ^ (r & 7u))) << 4);
 }
-__host__ __device__ constexpr uint32_t lds_swizzle_h(uint32_t r, uint32_t c) {  // c in 0..3
-  return ((r >> 2) << 8) | (((4u * (r & 3u)) + (c ^ ((r >> 2) & 3u))) << 4);
-}
 
 #define FFNK_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define FFNK_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
-
-constexpr int kBKH = 32;        // K elements per ring stage
-constexpr int kRowBytesH = 64;  // kBKH * sizeof(bf16)
-constexpr int kStages = 4;      // ring depth: one stage computing, one landed, two in flight
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool DUAL_, bool GATHER_A_, bool SCATTER_C_,
           bool DIRECT_, int GROUP_M_>
@@ -52,7 +42,7 @@ struct RoutedGemmCfg {
   static constexpr bool DUAL = DUAL_;
   static constexpr bool GATHER_A = GATHER_A_;
   static constexpr bool SCATTER_C = SCATTER_C_;
-  static constexpr bool DIRECT = DIRECT_;   // global->LDS loads bypass registers (needs K % 32 == 0)
+  static constexpr bool DIRECT = DIRECT_;   // global->LDS loads bypass registers (needs K % 64 == 0)
   static constexpr int GROUP_M = GROUP_M_;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int NT = NWAVES * kWave;
@@ -64,9 +54,7 @@ struct RoutedGemmCfg {
   static constexpr int TN = DUAL ? 2 * TN_OUT : TN_OUT;    // accumulator tiles per wave, N direction
   static constexpr int A_BYTES = BM * kRowBytes;           // slab layout
   static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
-  static constexpr int A_BYTES_H = BM * kRowBytesH;        // half-slab layout
-  static constexpr int STAGE_BYTES_H = (BM + BN) * kRowBytesH;
-  static constexpr int LDS_BYTES = DIRECT ? kStages * STAGE_BYTES_H : 2 * STAGE_BYTES;
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
   static_assert(WTM % 32 == 0 && WTN_OUT % 32 == 0, "wave tile must be a multiple of 32x32");
   static_assert(NWAVES % 2 == 0, "lane mapping of the slab layout needs an even wave count");
   static_assert((BM / 16) % NWAVES == 0 && (BN / 16) % NWAVES == 0, "panel rows must split evenly over waves");
@@ -90,35 +78,6 @@ __device__ __forceinline__ void zero_acc(f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 }
 
-// =============================================================================================
-// Direct path: 4-stage ring of 32-element K half-slabs, filled by buffer_load ... lds.
-// =============================================================================================
-// Which 16-byte chunks this lane moves.  A panel is moved as 1 KB groups of 16 rows x 64 bytes;
-// group id = j * NWAVES + wave; the lane fills physical slot `lane` of its group:
-//   lds_swizzle_h(group * 16 + r_in, c_log) == group * 1024 + lane * 16.
-template <class Cfg>
-struct RingLanes {
-  static constexpr int NJA = Cfg::BM / 16 / Cfg::NWAVES;
-  static constexpr int NJB = Cfg::BN / 16 / Cfg::NWAVES;
-  int lane, wave, wm, wn;
-  uint32_t r_in, c_log, lr, lh;
-  __device__ __forceinline__ void init() {
-    const int tid = threadIdx.x;
-    lane = tid & (kWave - 1);
-    wave = tid / kWave;
-    wm = wave / Cfg::WAVES_N;
-    wn = wave % Cfg::WAVES_N;
-    const uint32_t line = lane >> 4, slot = lane & 15;
-    r_in = 4 * line + (slot >> 2);
-    c_log = (slot & 3) ^ (line & 3);
-    lr = lane & 31;
-    lh = lane >> 5;
-  }
-  // First tile row of load group j of this wave (uniform over the wave), and this lane's row.
-  __device__ __forceinline__ int group_row(int j) const { return (j * Cfg::NWAVES + wave) * 16; }
-  __device__ __forceinline__ int load_row(int j) const { return group_row(j) + (int)r_in; }
-};
-
 constexpr int waitcnt_imm(int vm, int lgkm) {  // gfx9 s_waitcnt encoding, expcnt untouched
   return (vm & 15) | (7 << 4) | ((lgkm & 15) << 8) | ((vm >> 4) << 14);
 }
@@ -127,144 +86,15 @@ constexpr int waitcnt_imm(int vm, int lgkm) {  // gfx9 s_waitcnt encoding, expcn
 // have returned, then barrier.  Written with builtins (not a fence) so that younger loads stay
 // in flight across the barrier.
 template <int N>
-__device__ __forceinline__ void ring_wait_barrier() {
+__device__ __forceinline__ void dma_wait_barrier() {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(N, 0));
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 }
 
-// K loop of one tile on the ring.  Load j of the A panel reads 16 bytes at baseA[j] + offA[j]
-// (+ 64 bytes per half-slab); baseA[j] is uniform over the wave, offA[j] is this lane's 32-bit
-// byte offset.  Likewise for B.  k_len is a positive multiple of 32.
-//
-// Iteration i: [wait: half-slab i+1 landed everywhere, stage of i-1 free] [issue loads of i+3]
-// then the MFMAs of half-slab i, whose first fragments were read during iteration i-1, with
-// the LDS reads of its second K step, the reads of the first fragments of half-slab i+1 and
-// the global->LDS loads interleaved one per MFMA, so that the matrix pipe never waits for a
-// barrier or an LDS round trip.
-template <class Cfg>
-__device__ __forceinline__ void gemm_mainloop_ring(const RingLanes<Cfg>& rl,
-                                                   const uint16_t* const (&baseA)[RingLanes<Cfg>::NJA],
-                                                   const uint32_t (&offA)[RingLanes<Cfg>::NJA],
-                                                   const uint16_t* const (&baseB)[RingLanes<Cfg>::NJB],
-                                                   const uint32_t (&offB)[RingLanes<Cfg>::NJB], int k_len,
-                                                   uint8_t* lds, f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
-  constexpr int NJA = RingLanes<Cfg>::NJA, NJB = RingLanes<Cfg>::NJB;
-  constexpr int L = NJA + NJB;  // loads per wave per half-slab
-  constexpr int NS = kStages;
-  constexpr int STAGE = Cfg::STAGE_BYTES_H, A_BYTES = Cfg::A_BYTES_H;
-  constexpr int NM = TM * TN, ND = TM + TN;
-  const int wave = rl.wave;
-
-  // The panel bases are uniform over a wavefront (they depend on the wave index only), but where a
-  // base is selected per wave (gate or up weight of the SwiGLU kernels) the compiler cannot see that
-  // and wraps the load in a loop over distinct descriptors: pin those to scalar registers.
-  auto wave_uniform = [](const uint16_t* p) {
-    if (!Cfg::DUAL) return reinterpret_cast<void*>(const_cast<uint16_t*>(p));
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
-  };
-  __amdgpu_buffer_rsrc_t rsA[NJA], rsB[NJB];
-#pragma unroll
-  for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseA[j]), 0, 0xffffffff, 0x00020000);
-#pragma unroll
-  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
-
-  uint32_t koff[2];
-#pragma unroll
-  for (int s = 0; s < 2; ++s) koff[s] = lds_swizzle_h(rl.lr, 2 * s + rl.lh);
-  const uint32_t a_base = (uint32_t)(rl.wm * Cfg::WTM) * kRowBytesH;
-  uint32_t b_base[TN];
-#pragma unroll
-  for (int tn = 0; tn < TN; ++tn) b_base[tn] = A_BYTES + (uint32_t)b_frag_row<Cfg>(rl.wn, tn) * kRowBytesH;
-
-  zero_acc<Cfg>(acc);
-  const int nh = k_len / kBKH;
-
-  auto issue = [&](int stage, int ih) {
-    uint8_t* st = lds + stage * STAGE;
-    const int kb = ih * kRowBytesH;
-#pragma unroll
-    for (int j = 0; j < NJA; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[j], FFNK_LDS_PTR(st + (j * NWAVES + wave) * 1024), 16, offA[j], kb, 0, 0);
-#pragma unroll
-    for (int j = 0; j < NJB; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[j], FFNK_LDS_PTR(st + A_BYTES + (j * NWAVES + wave) * 1024), 16, offB[j], kb, 0, 0);
-  };
-  bf16x8_t fa[2][TM], fb[2][TN];
-  auto load_frags = [&](int buf, int stage, int s) {
-    const uint8_t* st = lds + stage * STAGE;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-      fa[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_base + i * 32 * kRowBytesH + koff[s]);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_base[j] + koff[s]);
-  };
-  auto mfmas = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        // D[n][m]: the weights are the MFMA "A" operand, so each lane ends up with runs of four
-        // consecutive output columns of one token row.
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
-  };
-
-  // Prologue: fill NS-1 stages, wait for the first, read its first fragments.
-#pragma unroll
-  for (int s = 0; s < NS - 1; ++s)
-    if (s < nh) issue(s, s);
-  if (nh > NS - 2) ring_wait_barrier<(NS - 2) * L>();
-  else ring_wait_barrier<0>();
-  load_frags(0, 0, 0);
-
-  auto body = [&](int u, int i, bool full) {
-    if (full || i + NS - 2 < nh) ring_wait_barrier<(NS - 3) * L>();
-    else ring_wait_barrier<0>();
-    if (full || i + NS - 1 < nh) issue((u + NS - 1) % NS, i + NS - 1);
-    load_frags(1, u, 1);
-    mfmas(0);
-    if (full || i + 1 < nh) load_frags(0, (u + 1) % NS, 0);
-    mfmas(1);
-    if (full) {
-      // Issue order inside the (branch-free) steady-state iteration: one LDS read after each of
-      // the first TM+TN MFMAs of a K step; the L global->LDS loads spread evenly over the MFMAs
-      // that follow in the two K steps (a load takes about two MFMA slots to issue).
-      constexpr int FREE = NM - ND;                     // MFMAs per K step without an LDS read
-      constexpr int GAP = (2 * FREE) / L > 0 ? (2 * FREE) / L : 1;
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-        for (int q = 0; q < NM; ++q) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (q < ND) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          else if ((ks * FREE + (q - ND)) % GAP == 0 && (ks * FREE + (q - ND)) / GAP < L)
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
-    }
-  };
-  int i0 = 0;
-  for (; i0 + 2 * NS - 2 < nh; i0 += NS) {  // every guard inside is true: no branches
-#pragma unroll
-    for (int u = 0; u < NS; ++u) body(u, i0 + u, true);
-  }
-  for (; i0 < nh; i0 += NS) {
-#pragma unroll
-    for (int u = 0; u < NS; ++u)
-      if (i0 + u < nh) body(u, i0 + u, false);
-  }
-#endif
-}
-
-// =============================================================================================
-// Register-staged path: 64-element K slabs, global -> registers -> LDS, double-buffered.  Handles
-// any K that is a multiple of 8 (chunks past the end are zero-filled).
-// =============================================================================================
+// Which 16-byte chunks a lane moves into LDS (both paths).  A panel is moved as 1 KB groups of
+// eight 128-byte rows; group id = j * NWAVES + wave; the lane fills physical slot `lane` of its group.
 template <class Cfg>
 struct TileLanes {
   static constexpr int NJA = Cfg::BM / 8 / Cfg::NWAVES;  // 1 KB (8-row) groups of the A panel per wave
@@ -288,10 +118,15 @@ struct TileLanes {
     lr = lane & 31;
     lh = lane >> 5;
   }
-  __device__ __forceinline__ int load_row(int j) const { return (j * Cfg::NWAVES + wave) * 8 + (int)r_in; }
+  __device__ __forceinline__ int group_row(int j) const { return (j * Cfg::NWAVES + wave) * 8; }
+  __device__ __forceinline__ int load_row(int j) const { return group_row(j) + (int)r_in; }
 };
 
-// pa[j] / pb[j] point at this lane's chunk of slab 0 for each of its rows; k_len % 8 == 0.
+// =============================================================================================
+// Register-staged path: 64-element K slabs, global -> registers -> LDS, double-buffered.  Handles
+// any K that is a multiple of 8 (chunks past the end are zero-filled).
+// pa[j] / pb[j] point at this lane's chunk of slab 0 for each of its rows.
+// =============================================================================================
 template <class Cfg>
 __device__ __forceinline__ void gemm_mainloop_staged(const TileLanes<Cfg>& tl,
                                                      const uint16_t* const (&pa)[TileLanes<Cfg>::NJA],
@@ -367,6 +202,130 @@ __device__ __forceinline__ void gemm_mainloop_staged(const TileLanes<Cfg>& tl,
       if (kt + 2 < nk) store_regs(lds0);
     }
   }
+}
+
+// =============================================================================================
+// Direct path: two stages of 64-element K slabs filled by buffer_load ... lds; k_len is a positive
+// multiple of 64.  Load j of the A panel reads 16 bytes at baseA[j] + offA[j] (+ 128 bytes per
+// slab); baseA[j] is uniform over the wave, offA[j] is this lane's 32-bit byte offset.  Likewise
+// for B.  Every load instruction moves eight whole 128-byte rows, so each cache line is requested
+// once (32-element half slabs cost a twentieth more time at d=4096, h=14336: the kernel runs at
+// the board's power limit, and the second request per line is paid for in shader clock).
+// One barrier per slab: it sits before the last K step, when every fragment of the current slab
+// has been read (its stage can be refilled with the slab after next) and the next slab, issued
+// one iteration earlier, has landed (its first fragments are read during the last K step).
+// =============================================================================================
+template <class Cfg>
+__device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
+                                                       const uint16_t* const (&baseA)[TileLanes<Cfg>::NJA],
+                                                       const uint32_t (&offA)[TileLanes<Cfg>::NJA],
+                                                       const uint16_t* const (&baseB)[TileLanes<Cfg>::NJB],
+                                                       const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
+                                                       uint8_t* lds, f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
+  constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
+  constexpr int L = NJA + NJB;
+  constexpr int STAGE = Cfg::STAGE_BYTES, A_BYTES = Cfg::A_BYTES;
+  constexpr int NM = TM * TN, ND = TM + TN;
+  const int wave = tl.wave;
+
+  auto wave_uniform = [](const uint16_t* p) {
+    if (!Cfg::DUAL) return reinterpret_cast<void*>(const_cast<uint16_t*>(p));
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+  };
+  __amdgpu_buffer_rsrc_t rsA[NJA], rsB[NJB];
+#pragma unroll
+  for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseA[j]), 0, 0xffffffff, 0x00020000);
+#pragma unroll
+  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
+
+  uint32_t koff[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) koff[s] = lds_swizzle(tl.lr, 2 * s + tl.lh);
+  const uint32_t a_base = (uint32_t)(tl.wm * Cfg::WTM) * kRowBytes;
+  uint32_t b_base[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) b_base[tn] = A_BYTES + (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
+
+  zero_acc<Cfg>(acc);
+  const int nk = k_len / kBK;
+
+  auto issue = [&](int stage, int kt) {
+    uint8_t* st = lds + stage * STAGE;
+    const int kb = kt * kRowBytes;
+#pragma unroll
+    for (int j = 0; j < NJA; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[j], FFNK_LDS_PTR(st + (j * NWAVES + wave) * 1024), 16, offA[j], kb, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NJB; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[j], FFNK_LDS_PTR(st + A_BYTES + (j * NWAVES + wave) * 1024), 16, offB[j], kb, 0, 0);
+  };
+  bf16x8_t fa[2][TM], fb[2][TN];
+  auto load_frags = [&](int buf, int stage, int s) {
+    const uint8_t* st = lds + stage * STAGE;
+    // In the order the MFMAs first use them: all weight fragments, then the token fragments.
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_base[j] + koff[s]);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      fa[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_base + i * 32 * kRowBytes + koff[s]);
+  };
+  auto mfmas = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+  };
+
+  issue(0, 0);
+  if (nk > 1) {
+    issue(1, 1);
+    dma_wait_barrier<L>();
+  } else {
+    dma_wait_barrier<0>();
+  }
+  load_frags(0, 0, 0);
+
+  auto body = [&](int u, int kt, bool full) {
+    load_frags(1, u, 1);
+    mfmas(0);
+    load_frags(0, u, 2);
+    mfmas(1);
+    load_frags(1, u, 3);
+    mfmas(0);
+    dma_wait_barrier<0>();
+    if (full || kt + 2 < nk) issue(u, kt + 2);
+    if (full || kt + 1 < nk) load_frags(0, u ^ 1, 0);
+    mfmas(1);
+    if (full) {
+      // One LDS read after each of the first TM+TN MFMAs of a K step; the global->LDS loads
+      // of the slab after next follow the barrier, spread over the MFMAs of the last K step.
+      constexpr int PER = (L + NM - 1) / NM;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int q = 0; q < NM; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (q < ND) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          if (ks == 3 && q * PER < L) __builtin_amdgcn_sched_group_barrier(0x020, PER, 0);
+        }
+    }
+  };
+  int k0 = 0;
+  for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches
+    body(0, k0, true);
+    body(1, k0 + 1, true);
+  }
+  for (; k0 < nk; k0 += 2) {
+    body(0, k0, false);
+    if (k0 + 1 < nk) body(1, k0 + 1, false);
+  }
+#endif
 }
 
 // Map a launch-order workgroup id to a position L in the tile order such that every XCD
@@ -471,8 +430,8 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
 
   f32x16_t acc[TM][TN];
   if (Cfg::DIRECT) {
-    constexpr int NJA = RingLanes<Cfg>::NJA, NJB = RingLanes<Cfg>::NJB;
-    RingLanes<Cfg> rl;
+    constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
+    TileLanes<Cfg> rl;
     rl.init();
     const uint16_t* baseA[NJA];
     uint32_t offA[NJA];
@@ -498,7 +457,7 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
       baseB[j] = (up ? g.B1[grp] : g.B0[grp]) + (int64_t)n_first * g.ldb;
       offB[j] = (uint32_t)(((int64_t)(n - n_first) * g.ldb + rl.c_log * 8) * 2);
     }
-    gemm_mainloop_ring<Cfg>(rl, baseA, offA, baseB, offB, g.K, lds, acc);
+    gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, g.K, lds, acc);
     routed_epilogue<Cfg>(g, acc, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
   } else {
     constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
@@ -526,12 +485,12 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
 }
 
 // Grouped split-K GEMM of the weight gradients (operands are padded to 64-element slabs, so
-// the ring path always applies).
+// the direct path always applies).
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArgs g) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
-  constexpr int NJA = RingLanes<Cfg>::NJA, NJB = RingLanes<Cfg>::NJB;
+  constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
   static_assert(!Cfg::DUAL && Cfg::DIRECT, "split-K GEMM runs on padded, 64-aligned slabs");
 
   __shared__ __attribute__((aligned(1024))) uint8_t lds[Cfg::LDS_BYTES];
@@ -561,7 +520,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
   const int64_t k_begin = (int64_t)k_begin_g + (int64_t)kt0 * kBK;
   const int k_len = (kt1 - kt0) * kBK;
 
-  RingLanes<Cfg> rl;
+  TileLanes<Cfg> rl;
   rl.init();
   const int r0 = tile_r * BN, c0 = tile_c * BM;
   f32x16_t acc[TM][TN];
@@ -583,7 +542,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
       baseB[j] = g.A + (int64_t)r_first * g.lda + k_begin;
       offB[j] = (uint32_t)(((int64_t)(r - r_first) * g.lda + rl.c_log * 8) * 2);
     }
-    gemm_mainloop_ring<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc);
+    gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc);
   } else {
     zero_acc<Cfg>(acc);  // a split without slabs (e.g. an empty modality) contributes exact zeros
   }

@@ -41,7 +41,9 @@ def test_workspace_bytes():
 def test_tile_table_entries():
     big = _lib.tile_config(_lib.OP_FFN_UP, 32768, 4096, 14336)
     assert big["path"] == _lib.PATH_MFMA_TILED and big["block_m"] == 256 and big["direct_lds"] == 1
-    assert big["block_k"] == 32 and big["lds_stages"] == 4  # direct global->LDS ring
+    assert big["block_k"] == 64 and big["lds_stages"] == 2  # two 64-element slabs, loaded global->LDS
+    half = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 96, 1024)
+    assert half["direct_lds"] == 0  # the direct path moves whole 128-byte lines: K % 64 == 0
     # M <= 8: dot-product streams, one wavefront per 1024-element K slice, no cross-workgroup split
     dec = _lib.tile_config(_lib.OP_FFN_FWD, 8, 4096, 14336)
     assert dec["path"] == _lib.PATH_STREAM and dec["lds_stages"] == 0 and dec["block_m"] == 8
