@@ -5,7 +5,7 @@
 
 namespace ffnk {
 
-constexpr int kGroupM = 8;  // M-tiles per L2 super-group in the tile order
+constexpr int kGroupM = 8;  // M-tiles per L2 super-group in the tile order (4 times the same, 16 costs 6 % at d=4096, h=14336)
 
 // Plain (single-weight) tiles: BN = output columns.
 template <bool GATHER, bool SCATTER, bool DIRECT>
@@ -36,10 +36,10 @@ inline hipError_t dispatch_tile(int tile, const GemmArgs& g, hipStream_t stream)
   }
 }
 
-// Plain GEMMs on the 256x256 tile: when the tile count is not a multiple of the CU count, the last
+// GEMMs on the 256x256 tile: when the tile count is not a multiple of the CU count, the last
 // round would run a few tiles on a few CUs for a full tile time (2064 tiles at M = 32768, N = 4096:
 // 8 rounds + 16 tiles).  Run the whole rounds with the big tile and the remainder as 128x128
-// tiles of the same schedule in a second launch.  Same K order per output element, so the result
+// tiles (128 rows x 64 gate + 64 up columns for the SwiGLU kernel) of the same schedule in a second launch.  Same K order per output element, so the result
 // does not depend on which launch computed it.
 template <class Tiles>
 inline hipError_t dispatch_tile_with_tail(int tile, const GemmArgs& g, hipStream_t stream) {

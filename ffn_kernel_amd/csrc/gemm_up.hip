@@ -4,7 +4,7 @@
 namespace ffnk {
 
 hipError_t launch_up_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream) {
-  return direct ? dispatch_tile<DualTiles<true>>(tile, g, stream)
+  return direct ? dispatch_tile_with_tail<DualTiles<true>>(tile, g, stream)
                 : dispatch_tile<DualTiles<false>>(tile, g, stream);
 }
 
