@@ -29,7 +29,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # profiles/ (routed_gemm_kernel_ffn_fwd_M32768_d4096_h14336.txt, stream_*_kernel_ffn_decode_*.txt).
 # Recorded, not measured live: counters cannot be read from inside the process.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg4": (9.4782e6 * 2.0 + 9.3048e5) * 1024,                                   # up-projection kernel
+    # up-projection: the whole-round launch plus the remainder launch (FETCH_SIZE * 2.0 + WRITE_SIZE each)
+    "cfg4": (5.4863e6 * 2.0 + 9.1223e5 + 2.3258e5 * 2.0 + 5388.9) * 1024,
     # decode: all launches of one call (up-projection, down-projection, reduce where there is one)
     "decode1v": (1.1476e5 * 2.0 + 40 + 5.7481e4 * 2.0 + 8) * 1024,
     "decode8": (2.2979e5 * 2.0 + 320 + 1.1568e5 * 2.0 + 64) * 1024,
@@ -216,7 +217,8 @@ def main() -> int:
         achieved = up_flops / (up_avg * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic,
-                    "kernel": "routed_gemm_kernel (up-projection + SwiGLU)", "kernel_ms": up_avg,
+                    "kernel": "routed_gemm_kernel (up-projection + SwiGLU: whole-round launch + remainder launch)",
+                    "kernel_ms": up_avg,
                     "down_kernel_ms": down_avg,
                     "down_achieved": 2 * M * w.d * w.h / (down_avg * 1e-3) / 1e12}
 
