@@ -149,6 +149,24 @@ int down_splits(int64_t M, int64_t d, int64_t h) {
   return stream_down_splits(d, h, stream_rows_per_block((int)M, false), stream_waves_per_block((int)M, false));
 }
 
+// Split-K factor of the down projection on the LDS-tiled path (1: none).
+// Tile and split-K factor of the down projection on the LDS-tiled path (a forced tile keeps its own
+// best split).
+RoutedPlan down_plan(int64_t M, int64_t d, int64_t h) {
+  RoutedPlan p;
+  if (g_force_tile >= 0 && g_force_tile < TILE_COUNT) {
+    p.tile = g_force_tile;
+    p.splits = pick_routed_splits(M, d, h, p.tile);
+  } else {
+    p = pick_routed_plan(M, d, h);
+  }
+  return p;
+}
+int down_tile(int64_t M, int64_t d, int64_t h) { return down_plan(M, d, h).tile; }
+int tiled_down_splits(int64_t M, int64_t d, int64_t h) {
+  return use_stream_path(M, d, h) ? 1 : down_plan(M, d, h).splits;
+}
+
 }  // namespace
 
 extern "C" {
@@ -176,10 +194,11 @@ size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
     case FFNK_OP_LINEAR_FWD:
       return route_ws_bytes(M);
     case FFNK_OP_FFN_FWD:
-      // perm + counts + the [M, h] bf16 intermediate in routed order (N = h); the streaming path
-      // adds the fp32 split-K partials of the down projection.
+      // perm + counts + the [M, h] bf16 intermediate in routed order (N = h) + the fp32 split-K
+      // partials of the down projection where it is split.
       return route_ws_bytes(M) + ws_align((size_t)M * round_up64(N, 8) * 2) +
-             (use_stream_path(M, K, N) ? ws_align((size_t)down_splits(M, K, N) * M * K * 4) : 0);
+             (use_stream_path(M, K, N) ? ws_align((size_t)down_splits(M, K, N) * M * K * 4)
+              : tiled_down_splits(M, K, N) > 1 ? ws_align((size_t)tiled_down_splits(M, K, N) * M * K * 4) : 0);
     case FFNK_OP_LINEAR_BWD: {
       const BwdPlan a = plan_bwd(M, K, N, true), b = plan_bwd(M, K, N, false);
       return a.total > b.total ? a.total : b.total;
@@ -209,7 +228,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
     case FFNK_OP_LINEAR_FWD: tile = pick_routed_tile(M, N, false); contraction = K; break;
     case FFNK_OP_FFN_FWD:
     case FFNK_OP_FFN_UP: tile = pick_routed_tile(M, N, true); dual = true; contraction = K; break;
-    case FFNK_OP_FFN_DOWN: tile = pick_routed_tile(M, K, false); contraction = N; break;  // out cols = d = K, contraction h = N
+    case FFNK_OP_FFN_DOWN: tile = down_plan(M, K, N).tile; contraction = N; break;  // out cols = d = K, contraction h = N
     case FFNK_OP_LINEAR_BWD:
     case FFNK_OP_BWD_DX: tile = pick_routed_tile(M, K, false); contraction = N; break;
     case FFNK_OP_BWD_DW: {
@@ -230,8 +249,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->group_m = 8;
   out->split_k = splits;
   out->direct_lds = (contraction > 0 && contraction % 64 == 0) ? 1 : 0;
-  out->block_k = 64;
-  out->lds_stages = 2;
+  if (op == FFNK_OP_FFN_DOWN && !stream) out->split_k = tiled_down_splits(M, K, N);
   if (stream) {
     // Streaming kernels: a workgroup is 16 * RT weight rows x one K range whose four wavefronts
     // take a quarter each; operands go global -> registers, no LDS staging.
@@ -409,7 +427,15 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
   dn.C = out; dn.ldc = out_stride_m;
   dn.perm = r.perm; dn.counts = r.counts;
   dn.M = (int)M; dn.N = (int)d; dn.K = (int)h;
-  FFNK_HIP(launch_down_gemm(routed_tile(M, d, false), direct_ok(h, 0, ldh, down_stride_n), dn, stream), "down-projection GEMM");
+  const bool dn_direct = direct_ok(h, 0, ldh, down_stride_n);
+  const int dn_splits = dn_direct ? tiled_down_splits(M, d, h) : 1;
+  if (dn_splits > 1) {
+    dn.splits = dn_splits;
+    dn.P = reinterpret_cast<float*>(wsb + r.bytes + ws_align((size_t)M * ldh * 2));
+  }
+  FFNK_HIP(launch_down_gemm(down_tile(M, d, h), dn_direct, dn, stream), "down-projection GEMM");
+  if (dn_splits > 1)
+    FFNK_HIP(launch_routed_reduce(dn.P, dn_splits, (int)M, (int)d, r.perm, out, out_stride_m, stream), "down-projection reduce");
   FFNK_HIP(mark(2), "event record");
   return FFNK_OK;
 }

@@ -21,6 +21,12 @@ struct GemmArgs {
   // remaining tiles, each cut into the kernel's own (smaller) tiles - launched with a smaller tile
   // config, this spreads the last, partial round over all CUs instead of leaving most of them idle.
   int sched_bm = 0, sched_bn = 0, tail_mode = 0;
+  // Split-K (direct path, tail_mode 0, not the SwiGLU kernels): with splits > 1 the contraction is
+  // cut into `splits` ranges of whole 64-element slabs, each workgroup handles one (tile, range) and
+  // stores its fp32 partial sums to P[split][routed row][N]; a reduce pass adds them and scatters
+  // the rows.  For outputs too small to fill the chip with tiles over a long contraction.
+  int splits = 1;
+  float* P = nullptr;
 };
 
 // Grouped split-K GEMM used for the weight gradients:

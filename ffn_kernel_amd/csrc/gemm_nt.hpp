@@ -380,6 +380,34 @@ __device__ __forceinline__ void routed_epilogue(const GemmArgs& g, f32x16_t (&ac
   }
 }
 
+// Split-K epilogue: fp32 partial sums of one K range, rows in routed order, no SwiGLU.
+template <class Cfg>
+__device__ __forceinline__ void routed_partial_store(const GemmArgs& g, f32x16_t (&acc)[Cfg::TM][Cfg::TN], int split,
+                                                     int row0, int row_end, int n0, int wm, int wn, uint32_t lr,
+                                                     uint32_t lh) {
+#pragma unroll
+  for (int i = 0; i < Cfg::TM; ++i) {
+    const int p = row0 + wm * Cfg::WTM + i * 32 + (int)lr;
+    if (p >= row_end) continue;
+    float* prow = g.P + ((int64_t)split * g.M + p) * g.N;
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int n = n0 + wn * Cfg::WTN_OUT + j * 32 + 8 * q4 + 4 * (int)lh;
+        if (n + 3 < g.N) {
+          *reinterpret_cast<float4*>(prow + n) =
+              make_float4(acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < g.N) prow[n + e] = acc[i][j][4 * q4 + e];
+        }
+      }
+    }
+  }
+}
+
 // Routed GEMM: rows in routed order, group-pure tiles.
 //   GATHER_A : A row of routed position p is perm[p] (else p)
 //   SCATTER_C: C row of routed position p is perm[p] (else p)
@@ -400,9 +428,13 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   const int tiles_m = tiles_v + cdiv(n_txt, SBM);
   const int tiles_n = cdiv(g.N, SBN);
   const int total = tiles_m * tiles_n;
-  int L, sub_m = 0, sub_n = 0;
+  int L, sub_m = 0, sub_n = 0, split = 0;
   if (g.tail_mode == 0) {
-    L = xcd_tile_slot(total);
+    L = xcd_tile_slot(total * g.splits);
+    if (g.splits > 1 && L >= 0) {  // range-major: neighbours in the order share panels, not a K range
+      split = L / total;
+      L -= split * total;
+    }
   } else {
     const int full = total / kCusPerChip * kCusPerChip;
     if (g.tail_mode == 1) {
@@ -433,13 +465,19 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
     constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
     TileLanes<Cfg> rl;
     rl.init();
+    // This workgroup's part of the contraction (all of it unless the launch splits K).
+    const int nk = g.K / kBK;
+    const int per_split = cdiv(nk, g.splits);
+    const int kt0 = min(split * per_split, nk);
+    const int k_len = (min(kt0 + per_split, nk) - kt0) * kBK;
+    const int64_t k0 = (int64_t)kt0 * kBK;
     const uint16_t* baseA[NJA];
     uint32_t offA[NJA];
     const uint16_t* baseB[NJB];
     uint32_t offB[NJB];
     // Gathered rows are addressed from the start of A (the host checks that 32 bits reach every
     // row); contiguous panels from their own first row.
-    const uint16_t* a0 = Cfg::GATHER_A ? g.A : g.A + (int64_t)row0 * g.lda;
+    const uint16_t* a0 = (Cfg::GATHER_A ? g.A : g.A + (int64_t)row0 * g.lda) + k0;
 #pragma unroll
     for (int j = 0; j < NJA; ++j) {
       int p = row0 + rl.load_row(j);
@@ -454,11 +492,13 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
       const int r = rl.load_row(j) - (up ? BN / 2 : 0);
       const int n_first = min(n0, g.N - 1);
       const int n = min(n0 + r, g.N - 1);
-      baseB[j] = (up ? g.B1[grp] : g.B0[grp]) + (int64_t)n_first * g.ldb;
+      baseB[j] = (up ? g.B1[grp] : g.B0[grp]) + (int64_t)n_first * g.ldb + k0;
       offB[j] = (uint32_t)(((int64_t)(n - n_first) * g.ldb + rl.c_log * 8) * 2);
     }
-    gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, g.K, lds, acc);
-    routed_epilogue<Cfg>(g, acc, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
+    if (k_len > 0) gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc);
+    else zero_acc<Cfg>(acc);  // a range past the end of K contributes exact zeros
+    if (!Cfg::DUAL && g.splits > 1) routed_partial_store<Cfg>(g, acc, split, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
+    else routed_epilogue<Cfg>(g, acc, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
   } else {
     constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
     TileLanes<Cfg> tl;
@@ -606,7 +646,8 @@ inline int routed_gemm_grid(int M, int N) {
 template <class Cfg>
 inline hipError_t launch_routed_gemm(const GemmArgs& g, hipStream_t stream) {
   if (g.M <= 0 || g.N <= 0) return hipSuccess;
-  const int grid = routed_gemm_grid<Cfg>(g.M, g.N);
+  if (g.splits > 1 && (Cfg::DUAL || !Cfg::DIRECT || g.tail_mode != 0 || g.P == nullptr)) return hipErrorInvalidValue;
+  const int grid = routed_gemm_grid<Cfg>(g.M, g.N) * (g.splits > 1 ? g.splits : 1);
   hipLaunchKernelGGL(routed_gemm_kernel<Cfg>, dim3(grid), dim3(Cfg::NT), 0, stream, g);
   return hipGetLastError();
 }

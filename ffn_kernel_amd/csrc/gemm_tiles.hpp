@@ -45,7 +45,7 @@ template <class Tiles>
 inline hipError_t dispatch_tile_with_tail(int tile, const GemmArgs& g, hipStream_t stream) {
   using Big = typename Tiles::T0;
   using Small = typename Tiles::T2;
-  if (tile != TILE_256x256_W8 || g.M <= 0 || g.N <= 0) return dispatch_tile<Tiles>(tile, g, stream);
+  if (tile != TILE_256x256_W8 || g.splits > 1 || g.M <= 0 || g.N <= 0) return dispatch_tile<Tiles>(tile, g, stream);
   GemmArgs a = g;
   a.tail_mode = 1;
   if (hipError_t e = launch_routed_gemm<Big>(a, stream)) return e;

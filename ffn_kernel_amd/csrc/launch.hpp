@@ -57,6 +57,10 @@ hipError_t launch_swiglu_bwd(uint16_t* T13, int64_t ld13, uint16_t* DH, int64_t 
 hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint16_t* out0, uint16_t* out1,
                                 int64_t sr, int64_t sc, hipStream_t stream);
 
+// out[perm[p], n] = bf16(sum_s P[s][p][n]): reduce pass of a split-K routed GEMM (N % 4 == 0, M < 65536).
+hipError_t launch_routed_reduce(const float* P, int splits, int M, int N, const int32_t* perm, uint16_t* out,
+                                int64_t ldo, hipStream_t stream);
+
 // ---- stream.hip: weight-streaming kernels for M <= 64 ----
 struct StreamArgs {
   const uint16_t* X; int64_t ldx;  // token rows: x [M, K] (gather_x = 1, token order) or H [M, K] (routed order)

@@ -217,4 +217,36 @@ hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint1
   return hipGetLastError();
 }
 
+// out[perm[p], n] = bf16(P[0][p][n] + P[1][p][n] + ...) in split order: the reduce pass of a split-K
+// routed GEMM.  One workgroup per (routed row, 1024 columns); N % 4 == 0.
+__global__ __launch_bounds__(256) void routed_reduce_kernel(const float* __restrict__ P, int splits, int M, int N,
+                                                            const int32_t* __restrict__ perm,
+                                                            uint16_t* __restrict__ out, int64_t ldo) {
+  const int p = blockIdx.y;
+  const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (n >= N) return;
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k = 0; k < splits; ++k) {
+    const float4 v = *reinterpret_cast<const float4*>(P + ((int64_t)k * M + p) * N + n);
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  uint16_t* o = out + (int64_t)perm[p] * ldo + n;
+  if ((reinterpret_cast<uintptr_t>(o) & 7) == 0) {
+    uint2 v2;
+    v2.x = pack2bf(s.x, s.y);
+    v2.y = pack2bf(s.z, s.w);
+    *reinterpret_cast<uint2*>(o) = v2;
+  } else {
+    o[0] = f2bf(s.x); o[1] = f2bf(s.y); o[2] = f2bf(s.z); o[3] = f2bf(s.w);
+  }
+}
+
+hipError_t launch_routed_reduce(const float* P, int splits, int M, int N, const int32_t* perm, uint16_t* out,
+                                int64_t ldo, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return hipSuccess;
+  dim3 grid((unsigned)cdiv(N, 1024), (unsigned)M);
+  hipLaunchKernelGGL(routed_reduce_kernel, grid, dim3(256), 0, stream, P, splits, M, N, perm, out, ldo);
+  return hipGetLastError();
+}
+
 }  // namespace ffnk

@@ -32,6 +32,70 @@ inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual) {
   return TILE_SMALL_W4;
 }
 
+// Tile and split-K factor of a routed GEMM with a single weight per group and a workspace for
+// partial sums (the FFN down projection).  When the output yields fewer tiles than the chip has
+// workgroup slots and the contraction is long, each workgroup would stream a long weight panel on
+// its own while most CUs idle; cutting K into `splits` ranges of whole 64-element slabs fills the
+// chip, at the price of fp32 partials (4 * splits * M * n_out bytes written, then read by the
+// reduce pass).  The choice minimises a cost model fitted to a sweep over M = 128 ... 4096 at
+// n_out = 4096, K = 14336 (it reproduces the measured best of every M there; the table's previous
+// choice was 1.1x to 1.7x slower):
+//   time = rounds * (5 us + slabs_per_range * t_slab) + splits * M * n_out * 8 bytes / 4 TB/s
+//   rounds = ceil(tiles * splits / slots),  slots = 256 CUs * workgroups per CU by LDS use,
+//   t_slab = 1.2 us for the 256x256 tile, 0.8 us for the 128x128 and 128x64 tiles.
+// Limited to M <= 4096 (above it the tiles fill the chip, and the reduce pass launches one row per
+// blockIdx.y); larger M keeps pick_routed_tile and no split.
+struct RoutedPlan {
+  int tile;
+  int splits;
+};
+
+inline double routed_plan_cost(int64_t M, int64_t n_out, int64_t K, int tile, int splits) {
+  const TileGeom t = tile_geom(tile, false);
+  const int64_t tiles = (cdiv64(M, t.block_m) + 1) * cdiv64(n_out, t.block_n_out);
+  const int64_t slots = (int64_t)kCus * (tile == TILE_SMALL_W4 ? 3 : tile == TILE_128x128_W4 ? 2 : 1);
+  const double t_slab = (tile == TILE_256x256_W8 || tile == TILE_256x256_W4) ? 1.2 : 0.8;
+  const int64_t slabs = cdiv64(cdiv64(K, 64), splits);
+  const double reduce = splits > 1 ? (double)splits * (double)M * (double)n_out * 8.0 / 4.0e6 : 0.0;
+  return (double)cdiv64(tiles * splits, slots) * (5.0 + (double)slabs * t_slab) + reduce;
+}
+
+// Best split for a given tile: ranges of at least 8 slabs, no empty range.
+inline int pick_routed_splits(int64_t M, int64_t n_out, int64_t K, int tile) {
+  if (M > 4096 || K % 64 != 0 || tile == TILE_256x256_W4) return 1;
+  const int64_t nk = K / 64;
+  int best = 1;
+  double best_cost = routed_plan_cost(M, n_out, K, tile, 1);
+  for (int s = 2; s <= 16 && nk / s >= 8; ++s) {
+    if (cdiv64(nk, cdiv64(nk, s)) != s) continue;  // would leave an empty range
+    const double c = routed_plan_cost(M, n_out, K, tile, s);
+    if (c < best_cost) {
+      best_cost = c;
+      best = s;
+    }
+  }
+  return best;
+}
+
+inline RoutedPlan pick_routed_plan(int64_t M, int64_t n_out, int64_t K) {
+  RoutedPlan p;
+  p.tile = pick_routed_tile(M, n_out, false);
+  p.splits = 1;
+  if (M > 4096 || K % 64 != 0) return p;
+  double best_cost = 0.0;
+  const int cand[3] = {TILE_256x256_W8, TILE_128x128_W4, TILE_SMALL_W4};
+  for (int i = 0; i < 3; ++i) {
+    const int s = pick_routed_splits(M, n_out, K, cand[i]);
+    const double c = routed_plan_cost(M, n_out, K, cand[i], s);
+    if (i == 0 || c < best_cost) {
+      best_cost = c;
+      p.tile = cand[i];
+      p.splits = s;
+    }
+  }
+  return p;
+}
+
 // Weight-gradient GEMM: two [R, Cc] outputs, contraction over about M / 2 rows each.
 inline TileChoice pick_splitk_tile(int64_t M, int64_t R, int64_t Cc) {
   TileChoice c;

@@ -175,7 +175,20 @@ FFN_SHAPES = [
     (333, 128, 320, 0.3),
     (2048, 1024, 2048, 0.5),
     (50, 36, 20, 0.5),        # generic path (d, h not multiples of 8)
+    # few output tiles over a long contraction: split-K down projection + reduce pass
+    (100, 256, 2048, 0.5),
+    (65, 1024, 2240, 0.4),    # 35 slabs: ranges of unequal length
+    (300, 512, 4096, 1.0),    # one modality only
+    (700, 264, 3072, 0.6),    # ragged output tile
 ]
+
+
+def test_ffn_fwd_split_k_table():
+    """The shapes above that are meant to exercise the split-K down projection do."""
+    for M, d, h in ((100, 256, 2048), (65, 1024, 2240), (300, 512, 4096), (700, 264, 3072)):
+        cfg = _lib.tile_config(_lib.OP_FFN_DOWN, M, d, h)
+        assert cfg["path"] == _lib.PATH_MFMA_TILED and cfg["split_k"] > 1, (M, d, h, cfg)
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 32768, 4096, 14336)["split_k"] == 1
 
 
 @pytest.mark.parametrize("M,d,h,p", FFN_SHAPES)
