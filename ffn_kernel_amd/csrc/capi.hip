@@ -162,6 +162,13 @@ RoutedPlan down_plan(int64_t M, int64_t d, int64_t h) {
   }
   return p;
 }
+// MaskedLinear forward: the table's tile unless cutting K pays (few output tiles, long contraction).
+RoutedPlan linear_plan(int64_t M, int64_t K, int64_t N) {
+  RoutedPlan p = down_plan(M, N, K);
+  if (N % 4 != 0) p.splits = 1;  // the reduce pass moves four columns per thread
+  if (p.splits == 1) p.tile = routed_tile(M, N, false);
+  return p;
+}
 int down_tile(int64_t M, int64_t d, int64_t h) { return down_plan(M, d, h).tile; }
 int tiled_down_splits(int64_t M, int64_t d, int64_t h) {
   return use_stream_path(M, d, h) ? 1 : down_plan(M, d, h).splits;
@@ -191,8 +198,11 @@ int ffnk_route(const uint8_t* mask, int64_t M, int32_t* perm, int32_t* counts, v
 size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
   if (M < 0 || K < 0 || N < 0 || M > kMaxRows || K > kMaxCols || N > kMaxCols) return (size_t)-1;
   switch (op) {
-    case FFNK_OP_LINEAR_FWD:
-      return route_ws_bytes(M);
+    case FFNK_OP_LINEAR_FWD: {
+      // perm + counts + the fp32 split-K partials where the GEMM is split
+      const int splits = linear_plan(M, K, N).splits;
+      return route_ws_bytes(M) + (splits > 1 ? ws_align((size_t)splits * M * N * 4) : 0);
+    }
     case FFNK_OP_FFN_FWD:
       // perm + counts + the [M, h] bf16 intermediate in routed order (N = h) + the fp32 split-K
       // partials of the down projection where it is split.
@@ -225,7 +235,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   int64_t contraction;
   int splits = 1;
   switch (op) {
-    case FFNK_OP_LINEAR_FWD: tile = pick_routed_tile(M, N, false); contraction = K; break;
+    case FFNK_OP_LINEAR_FWD: { const RoutedPlan lp = linear_plan(M, K, N); tile = lp.tile; splits = lp.splits; contraction = K; break; }
     case FFNK_OP_FFN_FWD:
     case FFNK_OP_FFN_UP: tile = pick_routed_tile(M, N, true); dual = true; contraction = K; break;
     case FFNK_OP_FFN_DOWN: tile = down_plan(M, K, N).tile; contraction = N; break;  // out cols = d = K, contraction h = N
@@ -308,7 +318,8 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
     FFNK_HIP(launch_generic_linear(a, stream), "generic linear kernel");
     return FFNK_OK;
   }
-  if (ws_bytes < route_ws_bytes(M) || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, route_ws_bytes(M));
+  const size_t need = ffnk_workspace_bytes(FFNK_OP_LINEAR_FWD, M, K, N);
+  if (ws_bytes < need || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, need);
   if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
   const RouteWs r = carve_route(static_cast<uint8_t*>(ws), M);
   FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
@@ -318,7 +329,19 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
   g.C = y; g.ldc = y_stride_m;
   g.perm = r.perm; g.counts = r.counts;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
-  FFNK_HIP(launch_linear_gemm(routed_tile(M, N, false), direct_ok(K, M, x_stride_m, w_stride_n), g, stream), "linear GEMM");
+  const bool direct = direct_ok(K, M, x_stride_m, w_stride_n);
+  RoutedPlan plan = linear_plan(M, K, N);
+  if (!direct) {
+    plan.splits = 1;
+    plan.tile = routed_tile(M, N, false);
+  }
+  if (plan.splits > 1) {
+    g.splits = plan.splits;
+    g.P = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + r.bytes);
+  }
+  FFNK_HIP(launch_linear_gemm(plan.tile, direct, g, stream), "linear GEMM");
+  if (plan.splits > 1)
+    FFNK_HIP(launch_routed_reduce(g.P, plan.splits, (int)M, (int)N, r.perm, y, y_stride_m, stream), "linear reduce");
   return FFNK_OK;
 }
 

@@ -71,6 +71,10 @@ LINEAR_SHAPES = [
     (2048, 1024, 1024, -1),          # cfg1 (span mask)
     (4096, 512, 2048, 0.5),          # 256x256 tile family
     (1000, 72, 264, 0.5),            # K % 64 != 0, K % 8 == 0
+    (24, 2048, 512, 0.5),            # few output tiles, long K: split-K + reduce pass
+    (1, 4096, 1024, 1.0),            # one row, split-K
+    (200, 3136, 260, 0.4),           # split-K with 49 slabs (unequal ranges), ragged N
+    (96, 1024, 250, 0.5),            # N % 4 != 0: no split
 ]
 
 
