@@ -162,6 +162,18 @@ RoutedPlan down_plan(int64_t M, int64_t d, int64_t h) {
   }
   return p;
 }
+// MaskedLinear forward at decode sizes: 0 = LDS-tiled GEMM, 1 = dot-product streams (M <= 8),
+// 2 = LDS-transposed streams (M <= 64).  The op is bound by reading each weight once.
+int linear_stream_kind(int64_t M, int64_t K, int64_t N) {
+  if (M < 1 || M > kStreamMaxM || K > kMaxCols || N > kMaxCols) return 0;
+  if (stream_dot_ok((int)M, (int)K)) return 1;
+  if (stream_tile_down_ok((int)M, (int)N, (int)K)) return 2;
+  return 0;
+}
+int linear_stream_splits(int64_t M, int64_t K, int64_t N) {
+  return linear_stream_kind(M, K, N) == 2 ? stream_tile_down_splits((int)M, (int)N, (int)K) : 1;
+}
+
 // MaskedLinear forward: the table's tile unless cutting K pays (few output tiles, long contraction).
 RoutedPlan linear_plan(int64_t M, int64_t K, int64_t N) {
   RoutedPlan p = down_plan(M, N, K);
@@ -199,8 +211,8 @@ size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
   if (M < 0 || K < 0 || N < 0 || M > kMaxRows || K > kMaxCols || N > kMaxCols) return (size_t)-1;
   switch (op) {
     case FFNK_OP_LINEAR_FWD: {
-      // perm + counts + the fp32 split-K partials where the GEMM is split
-      const int splits = linear_plan(M, K, N).splits;
+      // perm + counts + the fp32 split-K partials where the GEMM (or the streamed projection) is split
+      const int splits = linear_stream_kind(M, K, N) ? linear_stream_splits(M, K, N) : linear_plan(M, K, N).splits;
       return route_ws_bytes(M) + (splits > 1 ? ws_align((size_t)splits * M * N * 4) : 0);
     }
     case FFNK_OP_FFN_FWD:
@@ -260,6 +272,27 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->split_k = splits;
   out->direct_lds = (contraction > 0 && contraction % 64 == 0) ? 1 : 0;
   if (op == FFNK_OP_FFN_DOWN && !stream) out->split_k = tiled_down_splits(M, K, N);
+  if (op == FFNK_OP_LINEAR_FWD && linear_stream_kind(M, K, N)) {
+    out->path = FFNK_PATH_STREAM;
+    out->waves_m = out->waves_n = 1;
+    out->group_m = 1;
+    if (linear_stream_kind(M, K, N) == 1) {
+      out->block_m = (int)M;
+      out->block_n = stream_dot_rows_per_block((int)N, false, (int)K);
+      out->block_k = 512 * stream_dot_slices_per_wave((int)K);
+      out->split_k = (int)(K / out->block_k);
+      out->lds_stages = 0;
+      out->direct_lds = 0;
+    } else {
+      out->block_m = 16 * (int)cdiv64(M, 16);
+      out->block_n = stream_tile_rows_per_block((int)M, false);
+      out->block_k = 128;
+      out->lds_stages = stream_tile_depth((int)M);
+      out->direct_lds = stream_tile_direct((int)M);
+      out->split_k = linear_stream_splits(M, K, N);
+    }
+    return FFNK_OK;
+  }
   if (stream) {
     // Streaming kernels: a workgroup is 16 * RT weight rows x one K range whose four wavefronts
     // take a quarter each; operands go global -> registers, no LDS staging.
@@ -322,6 +355,24 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
   if (ws_bytes < need || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, need);
   if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
   const RouteWs r = carve_route(static_cast<uint8_t*>(ws), M);
+  if (const int kind = linear_stream_kind(M, K, N)) {
+    // Decode sizes: the weight-streaming kernels of the FFN's down projection, fed token rows in
+    // token order; they route from the mask themselves.
+    if (kind == 2 && M * x_stride_m >= ((int64_t)1 << 30))
+      return fail(FFNK_E_STRIDE, "x_stride_m=%lld: the decode kernels address the token rows with 32-bit offsets",
+                  (long long)x_stride_m);
+    const int splits = linear_stream_splits(M, K, N);
+    StreamArgs a;
+    a.X = x; a.ldx = x_stride_m; a.gather_x = 1; a.mask = mask; a.M = (int)M;
+    a.W0[0] = Wv; a.W0[1] = Wt; a.W1[0] = a.W1[1] = nullptr; a.ldw = w_stride_n;
+    a.Nrows = (int)N; a.K = (int)K; a.splits = splits; a.H = nullptr; a.ldh = 0;
+    a.P = splits > 1 ? reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + r.bytes) : nullptr;
+    a.out = y; a.ldo = y_stride_m;
+    FFNK_HIP(kind == 1 ? launch_stream_dot_down(a, stream) : launch_stream_tile_down(a, stream), "streaming linear");
+    if (splits > 1)
+      FFNK_HIP(launch_stream_reduce(a.P, splits, (int)M, (int)N, mask, y, y_stride_m, stream), "streaming reduce");
+    return FFNK_OK;
+  }
   FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
   GemmArgs g;
   g.A = x; g.lda = x_stride_m;

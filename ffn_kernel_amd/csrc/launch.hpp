@@ -88,6 +88,7 @@ hipError_t launch_stream_dot_up(const StreamArgs& a, hipStream_t stream);
 hipError_t launch_stream_dot_down(const StreamArgs& a, hipStream_t stream);
 // stream_tile.hip: 9 <= M <= 64, contiguous loads + LDS transpose + shared token-row slab.
 bool stream_tile_ok(int M, int d, int h);
+bool stream_tile_down_ok(int M, int Nrows, int K);  // single-weight projection alone (MaskedLinear forward)
 int stream_tile_rows_per_block(int M, bool dual);
 int stream_tile_depth(int M);
 int stream_tile_direct(int M);  // 1: the token-row slab is filled by direct global->LDS loads

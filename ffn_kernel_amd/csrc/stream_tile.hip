@@ -372,6 +372,12 @@ bool stream_tile_ok(int M, int d, int h) {
          h % stream_tile_rows_per_block(M, true) == 0 && d % stream_tile_rows_per_block(M, false) == 0;
 }
 
+// A single-weight projection (down projection, linear layer) of Nrows outputs over K on these kernels.
+bool stream_tile_down_ok(int M, int Nrows, int K) {
+  return M >= 1 && M <= kTMaxM && K % kTK == 0 && K / kTK >= kTMinChunks && Nrows > 0 &&
+         Nrows % stream_tile_rows_per_block(M, false) == 0;
+}
+
 // K split of the down projection: about one workgroup per CU and modality, at least eight chunks
 // per workgroup, every split non-empty.
 int stream_tile_down_splits(int M, int d, int h) {

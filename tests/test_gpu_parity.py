@@ -71,8 +71,15 @@ LINEAR_SHAPES = [
     (2048, 1024, 1024, -1),          # cfg1 (span mask)
     (4096, 512, 2048, 0.5),          # 256x256 tile family
     (1000, 72, 264, 0.5),            # K % 64 != 0, K % 8 == 0
-    (24, 2048, 512, 0.5),            # few output tiles, long K: split-K + reduce pass
-    (1, 4096, 1024, 1.0),            # one row, split-K
+    (100, 2048, 512, 0.5),           # few output tiles, long K: split-K + reduce pass
+    # decode sizes (M <= 64): the weight-streaming kernels of the FFN down projection
+    (1, 4096, 1024, 1.0),            # dot-product streams, one row
+    (8, 512, 100, 0.5),              # dot-product streams, ragged N, one slice
+    (5, 1024, 1000, 0.4),
+    (24, 2048, 512, 0.5),            # LDS-transposed streams, split-K + reduce
+    (40, 1024, 192, 0.5),            # eight chunks, no split
+    (64, 2048, 256, 0.5),
+    (33, 1152, 320, 0.0),            # nine chunks, one modality absent
     (200, 3136, 260, 0.4),           # split-K with 49 slabs (unequal ranges), ragged N
     (96, 1024, 250, 0.5),            # N % 4 != 0: no split
 ]
@@ -107,6 +114,26 @@ def test_linear_row_selection_is_exact(dev):
     y = MaskedLinear.apply(x.to(dev), eye.to(dev).T, (2 * eye).to(dev).T, mask.to(dev)).cpu()
     expect = torch.where(mask[:, None], x, 2 * x)
     assert torch.equal(y, expect)
+
+
+@pytest.mark.parametrize("M", [3, 17, 64])
+def test_linear_decode_rows_exact_and_absent_weight_untouched(dev, M):
+    """Decode sizes run on the weight-streaming kernels: identity weights select bit for bit, and the
+    weight of a modality with no rows is never read (NaN poison)."""
+    note(f"linear decode identity/poison M={M}")
+    K = 1024
+    gen = torch.Generator().manual_seed(M)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    mask = torch.rand(M, generator=gen) < 0.5
+    assert _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, K)["path"] == _lib.PATH_STREAM
+    eye = torch.eye(K).to(torch.bfloat16)
+    y = MaskedLinear.apply(x.to(dev), eye.to(dev).T, (2 * eye).to(dev).T, mask.to(dev)).cpu()
+    assert torch.equal(y, torch.where(mask[:, None], x, 2 * x))
+    poison = torch.full((K, K), float("nan"), dtype=torch.bfloat16)
+    y = MaskedLinear.apply(x.to(dev), eye.to(dev).T, poison.to(dev).T, torch.ones(M, dtype=torch.bool, device=dev)).cpu()
+    assert torch.equal(y, x)
+    y = MaskedLinear.apply(x.to(dev), poison.to(dev).T, eye.to(dev).T, torch.zeros(M, dtype=torch.bool, device=dev)).cpu()
+    assert torch.equal(y, x)
 
 
 def test_linear_unused_branch_never_touched(dev):
