@@ -136,6 +136,20 @@ def test_linear_decode_rows_exact_and_absent_weight_untouched(dev, M):
     assert torch.equal(y, x)
 
 
+@pytest.mark.parametrize("p", [1.0, 0.0, 0.5])
+def test_linear_decode_long_k_single_modality(dev, p):
+    """Streamed linear with 16-chunk K ranges: one modality absent or both present."""
+    M, K, N = 40, 8192, 4096
+    note(f"linear decode long K p={p}")
+    cfg = _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, N)
+    assert cfg["path"] == _lib.PATH_STREAM and cfg["split_k"] == 4
+    gen = torch.Generator().manual_seed(11)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_linear("t", M, K, N, mask, seed=5)
+    y = _run_linear(w, dev)
+    assert_close(y, om.linear_select(w.x, w.Wv, w.Wt, w.mask, torch.float64), f"linear decode long K p={p}")
+
+
 def test_linear_unused_branch_never_touched(dev):
     """Poisoning the text weight with NaN must leave visual rows finite (the blend form would not)."""
     note("linear NaN poison")
@@ -307,6 +321,25 @@ def test_ffn_decode_tile_stream_vs_oracle(dev, M, kind, d, h):
     torch.cuda.synchronize()
     assert_close(out, cref.ffn_fwd(w.x, w.W, w.mask, round_mid=True), f"decode tile stream {M} {kind}")
     if kind in ("visual", "text"):
+        W = dict(w.W)
+        for k in (("u1", "u2", "u3") if kind == "visual" else ("w1", "w2", "w3")):
+            W[k] = torch.full_like(W[k], float("nan"))
+        out2 = MaskedFFN.apply(*wl.FFNWorkload("p", w.x, W, w.mask).to(dev).op_args())
+        assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("kind", ["visual", "text", "bernoulli"])
+def test_ffn_decode_long_ranges(dev, kind):
+    """Decode call whose down projection is split into K ranges of 16 chunks; one modality absent or
+    both present, and the absent modality's weights are never read."""
+    M, d, h = 48, 4096, 8192
+    note(f"ffn decode long ranges M={M} kind={kind}")
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, M, d, h)["split_k"] == 4  # 16 chunks per range
+    w = wl.cfg5_ffn_decode(M, kind, seed=7, d=d, h=h)
+    out = MaskedFFN.apply(*w.to(dev).op_args())
+    torch.cuda.synchronize()
+    assert_close(out, om.ffn_select(w.x, w.W, w.mask, torch.float64, round_intermediate=True), f"long ranges {kind}")
+    if kind != "bernoulli":
         W = dict(w.W)
         for k in (("u1", "u2", "u3") if kind == "visual" else ("w1", "w2", "w3")):
             W[k] = torch.full_like(W[k], float("nan"))
