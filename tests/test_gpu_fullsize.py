@@ -53,15 +53,23 @@ def test_cfg4_rows_against_c_oracle(cfg4):
 
 
 def test_cfg4_batch_composition_invariance(dev, cfg4):
-    """A row's result does not depend on which other rows share the call: one sequence alone (another
-    tile schedule, same K order) reproduces its rows of the full call bit for bit."""
+    """A row's result does not depend on which other rows share the call: two sequences alone (another
+    tile schedule, same K order) reproduce their rows of the full call bit for bit.  A single sequence
+    (4096 rows) runs its down projection split over K, i.e. in another summation order: equal to
+    bf16 accuracy."""
     note("cfg4 batch invariance")
     w, d, out = cfg4
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 8192, w.d, w.h)["split_k"] == 1
     for seq in (0, 5):
-        sl = slice(seq * 4096, (seq + 1) * 4096)
+        sl = slice(seq * 4096, (seq + 2) * 4096)
         sub = wl.FFNWorkload("seq", d.x[sl].contiguous(), d.W, d.mask[sl].contiguous())
         part = MaskedFFN.apply(*sub.op_args())
         assert torch.equal(part, out[sl])
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 4096, w.d, w.h)["split_k"] > 1
+    sl = slice(3 * 4096, 4 * 4096)
+    sub = wl.FFNWorkload("seq", d.x[sl].contiguous(), d.W, d.mask[sl].contiguous())
+    part = MaskedFFN.apply(*sub.op_args())
+    assert_close_bf16_pair(part, out[sl].float().cpu(), "one sequence (split-K down projection) vs the full call")
 
 
 def test_cfg4_uniform_sequences_against_library_matmul(dev, cfg4):
