@@ -664,7 +664,21 @@ int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x
   b.B0[0] = w13[0]; b.B0[1] = w13[1]; b.B1[0] = b.B1[1] = nullptr; b.ldb = ld13;
   b.C = dx; b.ldc = dx_stride_m; b.perm = r.perm; b.counts = r.counts;
   b.M = (int)M; b.N = (int)d; b.K = (int)(2 * h);
-  FFNK_HIP(launch_down_gemm(routed_tile(M, d, false), direct_ok(2 * h, 0, ld13, ld13), b, stream), "dx GEMM");
+  // Few output tiles over a 2h-long contraction: split K like the forward's down projection.  The
+  // fp32 partials live where the W2^T copies were (dead since the dh GEMM), if they fit there.
+  const bool dx_direct = direct_ok(2 * h, 0, ld13, ld13);
+  RoutedPlan dxp = down_plan(M, d, 2 * h);
+  if (!dx_direct || (size_t)dxp.splits * M * d * 4 > 2 * ws_align((size_t)h * d * 2)) {
+    dxp.splits = 1;
+    dxp.tile = routed_tile(M, d, false);
+  }
+  if (dxp.splits > 1) {
+    b.splits = dxp.splits;
+    b.P = reinterpret_cast<float*>(wsb + p.off_w2t);
+  }
+  FFNK_HIP(launch_down_gemm(dxp.tile, dx_direct, b, stream), "dx GEMM");
+  if (dxp.splits > 1)
+    FFNK_HIP(launch_routed_reduce(b.P, dxp.splits, (int)M, (int)d, r.perm, dx, dx_stride_m, stream), "dx reduce");
 
   // ---- weight gradients: contraction over the rows of each group, on 64-padded transposes ----
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);    // [d, ldt]

@@ -394,6 +394,7 @@ FFN_BWD_SHAPES = [
     (300, 256, 512, 0.5),
     (1000, 512, 384, 0.3),
     (2048, 1024, 2048, 0.5),
+    (150, 256, 1024, 0.5),  # dx GEMM: few output tiles over a 2048-long contraction, split over K
 ]
 
 
