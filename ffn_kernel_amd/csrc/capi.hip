@@ -9,6 +9,7 @@
 #include "common.hpp"
 #include "launch.hpp"
 #include "tile_table.hpp"
+#include "gemm_sched.hpp"
 
 using namespace ffnk;
 
@@ -185,6 +186,14 @@ int down_tile(int64_t M, int64_t d, int64_t h) { return down_plan(M, d, h).tile;
 int tiled_down_splits(int64_t M, int64_t d, int64_t h) {
   return use_stream_path(M, d, h) ? 1 : down_plan(M, d, h).splits;
 }
+// fp32 partials of the tiled down projection: all rows when K is split for the whole GEMM, or the
+// kTailSlots tiles of the split tail when the 256x256 tile runs unsplit.
+size_t tiled_down_partial_bytes(int64_t M, int64_t d, int64_t h) {
+  const RoutedPlan p = down_plan(M, d, h);
+  if (p.splits > 1) return ws_align((size_t)p.splits * M * d * 4);
+  if (p.tile == TILE_256x256_W8 && h % 64 == 0) return ws_align((size_t)kTailSlots * 256 * 256 * 4);
+  return 0;
+}
 
 }  // namespace
 
@@ -219,8 +228,7 @@ size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
       // perm + counts + the [M, h] bf16 intermediate in routed order (N = h) + the fp32 split-K
       // partials of the down projection where it is split.
       return route_ws_bytes(M) + ws_align((size_t)M * round_up64(N, 8) * 2) +
-             (use_stream_path(M, K, N) ? ws_align((size_t)down_splits(M, K, N) * M * K * 4)
-              : tiled_down_splits(M, K, N) > 1 ? ws_align((size_t)tiled_down_splits(M, K, N) * M * K * 4) : 0);
+             (use_stream_path(M, K, N) ? ws_align((size_t)down_splits(M, K, N) * M * K * 4) : tiled_down_partial_bytes(M, K, N));
     case FFNK_OP_LINEAR_BWD: {
       const BwdPlan a = plan_bwd(M, K, N, true), b = plan_bwd(M, K, N, false);
       return a.total > b.total ? a.total : b.total;
@@ -503,9 +511,12 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
   dn.M = (int)M; dn.N = (int)d; dn.K = (int)h;
   const bool dn_direct = direct_ok(h, 0, ldh, down_stride_n);
   const int dn_splits = dn_direct ? tiled_down_splits(M, d, h) : 1;
+  float* partials = reinterpret_cast<float*>(wsb + r.bytes + ws_align((size_t)M * ldh * 2));
   if (dn_splits > 1) {
     dn.splits = dn_splits;
-    dn.P = reinterpret_cast<float*>(wsb + r.bytes + ws_align((size_t)M * ldh * 2));
+    dn.P = partials;
+  } else if (dn_direct && down_tile(M, d, h) == TILE_256x256_W8) {
+    dn.P_tail = partials;  // the last, partial round of 256x256 tiles runs cut into K ranges
   }
   FFNK_HIP(launch_down_gemm(down_tile(M, d, h), dn_direct, dn, stream), "down-projection GEMM");
   if (dn_splits > 1)

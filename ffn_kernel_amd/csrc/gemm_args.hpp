@@ -20,6 +20,8 @@ struct GemmArgs {
   // that fill whole rounds of the chip (the first floor(tiles / 256) * 256 of the order).  2: only the
   // remaining tiles, each cut into the kernel's own (smaller) tiles - launched with a smaller tile
   // config, this spreads the last, partial round over all CUs instead of leaving most of them idle.
+  // 3: only the remaining tiles, on the kernel's own tile, each cut into K ranges (split tail, see
+  // P_tail below).
   int sched_bm = 0, sched_bn = 0, tail_mode = 0;
   // Split-K (direct path, tail_mode 0, not the SwiGLU kernels): with splits > 1 the contraction is
   // cut into `splits` ranges of whole 64-element slabs, each workgroup handles one (tile, range) and
@@ -27,6 +29,12 @@ struct GemmArgs {
   // the rows.  For outputs too small to fill the chip with tiles over a long contraction.
   int splits = 1;
   float* P = nullptr;
+  // Split tail (direct path, single weight per group): the launcher runs the whole rounds of 256 tiles
+  // first and then the remaining tiles cut into tail_split_factor() K ranges each, so that the last,
+  // partial round takes a fraction of a tile time.  P_tail holds kTailSlots fp32 tiles of the
+  // kernel's macro tile; a reduce pass adds the ranges and scatters the rows.  NULL: the remainder
+  // runs as smaller tiles over all of K (tail_mode 2).
+  float* P_tail = nullptr;
 };
 
 // Grouped split-K GEMM used for the weight gradients:

@@ -12,6 +12,7 @@
 #pragma once
 #include "common.hpp"
 #include "gemm_args.hpp"
+#include "gemm_sched.hpp"
 
 namespace ffnk {
 
@@ -30,7 +31,6 @@ __host__ __device__ constexpr uint32_t lds_swizzle(uint32_t r, uint32_t c) {  //
 }
 
 #define FFNK_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-#define FFNK_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool DUAL_, bool GATHER_A_, bool SCATTER_C_,
           bool DIRECT_, int GROUP_M_>
@@ -331,7 +331,6 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
 // Map a launch-order workgroup id to a position L in the tile order such that every XCD
 // (workgroup b runs on XCD b % 8) owns one contiguous range of the order: tiles that share
 // A rows / B columns then meet in the same L2.  Returns -1 for a surplus workgroup.
-constexpr int kCusPerChip = 256;
 
 __device__ __forceinline__ int xcd_tile_slot(int total) {
   const int per_xcd = cdiv(total, kXcds);
@@ -380,16 +379,17 @@ __device__ __forceinline__ void routed_epilogue(const GemmArgs& g, f32x16_t (&ac
   }
 }
 
-// Split-K epilogue: fp32 partial sums of one K range, rows in routed order, no SwiGLU.
+// Split-K epilogue: fp32 partial sums of one K range, no SwiGLU.  Element (routed row p, column n)
+// goes to base[p * ld + n].
 template <class Cfg>
-__device__ __forceinline__ void routed_partial_store(const GemmArgs& g, f32x16_t (&acc)[Cfg::TM][Cfg::TN], int split,
-                                                     int row0, int row_end, int n0, int wm, int wn, uint32_t lr,
-                                                     uint32_t lh) {
+__device__ __forceinline__ void routed_partial_store(float* base, int64_t ld, const GemmArgs& g,
+                                                     f32x16_t (&acc)[Cfg::TM][Cfg::TN], int row0, int row_end, int n0,
+                                                     int wm, int wn, uint32_t lr, uint32_t lh) {
 #pragma unroll
   for (int i = 0; i < Cfg::TM; ++i) {
     const int p = row0 + wm * Cfg::WTM + i * 32 + (int)lr;
     if (p >= row_end) continue;
-    float* prow = g.P + ((int64_t)split * g.M + p) * g.N;
+    float* prow = base + (int64_t)p * ld;
 #pragma unroll
     for (int j = 0; j < Cfg::TN; ++j) {
 #pragma unroll
@@ -423,15 +423,12 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   const int SBM = g.sched_bm > 0 ? g.sched_bm : BM;
   const int SBN = g.sched_bn > 0 ? g.sched_bn : Cfg::BN_OUT;
   const int n_vis = g.counts[0];
-  const int n_txt = g.M - n_vis;
-  const int tiles_v = cdiv(n_vis, SBM);
-  const int tiles_m = tiles_v + cdiv(n_txt, SBM);
-  const int tiles_n = cdiv(g.N, SBN);
-  const int total = tiles_m * tiles_n;
-  int L, sub_m = 0, sub_n = 0, split = 0;
+  const int total = routed_tile_count(n_vis, g.M, g.N, SBM, SBN);
+  int L, sub_m = 0, sub_n = 0, split = 0, splits = 1, tail_slot = 0;
   if (g.tail_mode == 0) {
-    L = xcd_tile_slot(total * g.splits);
-    if (g.splits > 1 && L >= 0) {  // range-major: neighbours in the order share panels, not a K range
+    splits = g.splits;
+    L = xcd_tile_slot(total * splits);
+    if (splits > 1 && L >= 0) {  // range-major: neighbours in the order share panels, not a K range
       split = L / total;
       L -= split * total;
     }
@@ -439,25 +436,27 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
     const int full = total / kCusPerChip * kCusPerChip;
     if (g.tail_mode == 1) {
       L = xcd_tile_slot(full);
-    } else {
+    } else if (g.tail_mode == 2) {
       const int qn = SBN / Cfg::BN_OUT, q = (SBM / BM) * qn;  // own tiles per macro tile
       if ((int)blockIdx.x >= (total - full) * q) return;
       L = full + (int)blockIdx.x / q;
       sub_m = ((int)blockIdx.x % q) / qn;
       sub_n = ((int)blockIdx.x % q) % qn;
+    } else {
+      const int n_tail = total - full;
+      splits = tail_split_factor(n_tail, g.K / kBK);
+      tail_slot = (int)blockIdx.x;
+      if (tail_slot >= n_tail * splits) return;
+      split = tail_slot / n_tail;
+      L = full + tail_slot % n_tail;
     }
   }
   if (L < 0) return;
-  const int width = Cfg::GROUP_M * tiles_n;
-  const int first_m = (L / width) * Cfg::GROUP_M;
-  const int gsz = min(Cfg::GROUP_M, tiles_m - first_m);
-  const int tile_m = first_m + (L % width) % gsz;
-  const int tile_n = (L % width) / gsz;
-
-  const int grp = tile_m < tiles_v ? 0 : 1;
-  const int row0 = (grp == 0 ? tile_m * SBM : n_vis + (tile_m - tiles_v) * SBM) + sub_m * BM;  // routed position
-  const int row_end = grp == 0 ? n_vis : g.M;
-  const int n0 = tile_n * SBN + sub_n * Cfg::BN_OUT;
+  const TileCoord tc = routed_tile_coord(L, n_vis, g.M, g.N, SBM, SBN, Cfg::GROUP_M);
+  const int grp = tc.grp;
+  const int row0 = tc.row0 + sub_m * BM;  // routed position
+  const int row_end = tc.row_end;
+  const int n0 = tc.n0 + sub_n * Cfg::BN_OUT;
   if (row0 >= row_end || n0 >= g.N) return;  // a sub-tile past the edge of a partial macro tile
 
   f32x16_t acc[TM][TN];
@@ -467,7 +466,7 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
     rl.init();
     // This workgroup's part of the contraction (all of it unless the launch splits K).
     const int nk = g.K / kBK;
-    const int per_split = cdiv(nk, g.splits);
+    const int per_split = cdiv(nk, splits);
     const int kt0 = min(split * per_split, nk);
     const int k_len = (min(kt0 + per_split, nk) - kt0) * kBK;
     const int64_t k0 = (int64_t)kt0 * kBK;
@@ -497,8 +496,15 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
     }
     if (k_len > 0) gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc);
     else zero_acc<Cfg>(acc);  // a range past the end of K contributes exact zeros
-    if (!Cfg::DUAL && g.splits > 1) routed_partial_store<Cfg>(g, acc, split, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
-    else routed_epilogue<Cfg>(g, acc, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
+    if (!Cfg::DUAL && splits > 1) {
+      if (g.tail_mode == 3)  // one compact fp32 tile per (tile, range) pair
+        routed_partial_store<Cfg>(g.P_tail + (int64_t)tail_slot * (BM * Cfg::BN_OUT) - ((int64_t)row0 * Cfg::BN_OUT + n0),
+                                  Cfg::BN_OUT, g, acc, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
+      else
+        routed_partial_store<Cfg>(g.P + (int64_t)split * g.M * g.N, g.N, g, acc, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
+    } else {
+      routed_epilogue<Cfg>(g, acc, row0, row_end, n0, rl.wm, rl.wn, rl.lr, rl.lh);
+    }
   } else {
     constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
     TileLanes<Cfg> tl;

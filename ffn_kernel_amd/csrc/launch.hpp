@@ -61,6 +61,11 @@ hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint1
 hipError_t launch_routed_reduce(const float* P, int splits, int M, int N, const int32_t* perm, uint16_t* out,
                                 int64_t ldo, hipStream_t stream);
 
+// Reduce pass of a split tail (GemmArgs::P_tail) of a GEMM on bm x bn tiles with scatter epilogue.
+hipError_t launch_routed_tail_reduce(const float* P_tail, int M, int N, int K, const int32_t* counts,
+                                     const int32_t* perm, int bm, int bn, int group_m, uint16_t* C, int64_t ldc,
+                                     hipStream_t stream);
+
 // ---- stream.hip: weight-streaming kernels for M <= 64 ----
 struct StreamArgs {
   const uint16_t* X; int64_t ldx;  // token rows: x [M, K] (gather_x = 1, token order) or H [M, K] (routed order)

@@ -4,6 +4,7 @@
 // K-contiguous form the MFMA core wants.
 #include "common.hpp"
 #include "launch.hpp"
+#include "gemm_sched.hpp"
 
 namespace ffnk {
 
@@ -246,6 +247,62 @@ hipError_t launch_routed_reduce(const float* P, int splits, int M, int N, const 
   if (M <= 0 || N <= 0) return hipSuccess;
   dim3 grid((unsigned)cdiv(N, 1024), (unsigned)M);
   hipLaunchKernelGGL(routed_reduce_kernel, grid, dim3(256), 0, stream, P, splits, M, N, perm, out, ldo);
+  return hipGetLastError();
+}
+
+// Reduce pass of a split tail (see GemmArgs::P_tail): workgroups (i, 0 .. kTailRowChunks - 1) add the K
+// ranges of tail tile i, one band of rows each, and scatter the rows, C[perm[p], n] = bf16(sum_k P_tail[k * n_tail + i][p - row0][n - n0]).
+// Recomputes the GEMM kernel's schedule from counts[]; exits when the tail was not split.
+constexpr int kTailRowChunks = 16;  // row bands per tile in the tail reduce: enough workgroups to fill the chip from 16 tiles
+
+__global__ __launch_bounds__(256) void routed_tail_reduce_kernel(const float* __restrict__ P_tail, int M, int N, int K,
+                                                                 const int32_t* __restrict__ counts,
+                                                                 const int32_t* __restrict__ perm, int bm, int bn,
+                                                                 int group_m, uint16_t* __restrict__ C, int64_t ldc) {
+  const int n_vis = counts[0];
+  const int total = routed_tile_count(n_vis, M, N, bm, bn);
+  const int full = total / kCusPerChip * kCusPerChip;
+  const int n_tail = total - full;
+  const int tile_i = blockIdx.x;
+  if (tile_i >= n_tail) return;
+  const int splits = tail_split_factor(n_tail, K / 64);
+  if (splits == 1) return;  // the GEMM stored this tile itself
+  const TileCoord tc = routed_tile_coord(full + tile_i, n_vis, M, N, bm, bn, group_m);
+  const int quads = bn / 4;                   // float4 columns per tile row
+  const int rows_per_pass = 256 / quads;
+  const int q = threadIdx.x % quads;
+  const int n = tc.n0 + 4 * q;
+  if (n >= N) return;
+  const int64_t tile_elems = (int64_t)bm * bn;
+  const int band = bm / kTailRowChunks;
+  for (int r = blockIdx.y * band + threadIdx.x / quads; r < (blockIdx.y + 1) * band; r += rows_per_pass) {
+    const int p = tc.row0 + r;
+    if (p >= tc.row_end) break;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k = 0; k < splits; ++k) {
+      const float4 v = *reinterpret_cast<const float4*>(P_tail + ((int64_t)k * n_tail + tile_i) * tile_elems + (int64_t)r * bn + 4 * q);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    uint16_t* o = C + (int64_t)perm[p] * ldc + n;
+    if (n + 3 < N && (reinterpret_cast<uintptr_t>(o) & 7) == 0) {
+      uint2 v2;
+      v2.x = pack2bf(s.x, s.y);
+      v2.y = pack2bf(s.z, s.w);
+      *reinterpret_cast<uint2*>(o) = v2;
+    } else {
+      const float e[4] = {s.x, s.y, s.z, s.w};
+      for (int i = 0; i < 4; ++i)
+        if (n + i < N) o[i] = f2bf(e[i]);
+    }
+  }
+}
+
+hipError_t launch_routed_tail_reduce(const float* P_tail, int M, int N, int K, const int32_t* counts,
+                                     const int32_t* perm, int bm, int bn, int group_m, uint16_t* C, int64_t ldc,
+                                     hipStream_t stream) {
+  if (M <= 0 || N <= 0 || bn % 4 != 0 || 256 % (bn / 4) != 0 || bm % kTailRowChunks != 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(routed_tail_reduce_kernel, dim3(kTailSlots, kTailRowChunks), dim3(256), 0, stream, P_tail, M, N, K, counts, perm, bm,
+                     bn, group_m, C, ldc);
   return hipGetLastError();
 }
 

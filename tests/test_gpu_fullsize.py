@@ -54,9 +54,10 @@ def test_cfg4_rows_against_c_oracle(cfg4):
 
 def test_cfg4_batch_composition_invariance(dev, cfg4):
     """A row's result does not depend on which other rows share the call: two sequences alone (another
-    tile schedule, same K order) reproduce their rows of the full call bit for bit.  A single sequence
-    (4096 rows) runs its down projection split over K, i.e. in another summation order: equal to
-    bf16 accuracy."""
+    tile schedule) reproduce their rows of the full call - bit for bit wherever the K order is shared,
+    i.e. everywhere except the few tiles of a call's last, partial round, which are summed in K ranges;
+    those and a single sequence (4096 rows, whose whole down projection is split over K) agree to bf16
+    accuracy."""
     note("cfg4 batch invariance")
     w, d, out = cfg4
     assert _lib.tile_config(_lib.OP_FFN_DOWN, 8192, w.d, w.h)["split_k"] == 1
@@ -64,7 +65,9 @@ def test_cfg4_batch_composition_invariance(dev, cfg4):
         sl = slice(seq * 4096, (seq + 2) * 4096)
         sub = wl.FFNWorkload("seq", d.x[sl].contiguous(), d.W, d.mask[sl].contiguous())
         part = MaskedFFN.apply(*sub.op_args())
-        assert torch.equal(part, out[sl])
+        same_rows = (part == out[sl]).all(dim=1).float().mean().item()
+        assert same_rows >= 0.9, same_rows
+        assert_close_bf16_pair(part, out[sl].float().cpu(), "two sequences vs the full call")
     assert _lib.tile_config(_lib.OP_FFN_DOWN, 4096, w.d, w.h)["split_k"] > 1
     sl = slice(3 * 4096, 4 * 4096)
     sub = wl.FFNWorkload("seq", d.x[sl].contiguous(), d.W, d.mask[sl].contiguous())
@@ -90,6 +93,31 @@ def test_cfg4_uniform_sequences_against_library_matmul(dev, cfg4):
         assert_close(out[seq * 4096:(seq + 1) * 4096], ref.double().cpu(), f"uniform sequence {seq}")
         checked += 1
     assert checked >= 2
+
+
+def test_ffn_split_tail_of_the_down_projection(dev):
+    """8500 rows x 4096 output columns: 34 or 35 row tiles x 16 column tiles of 256x256, i.e. two whole
+    rounds of 256 tiles and a remainder that runs cut into K ranges with a reduce pass.  Checked against
+    fp32 library matmuls of the select form on the GPU (every row, so the remainder's rows are covered)."""
+    note("ffn split tail M=8500 d=4096 h=1024")
+    M, d, h = 8500, 4096, 1024
+    cfg = _lib.tile_config(_lib.OP_FFN_DOWN, M, d, h)
+    assert cfg["block_m"] == 256 and cfg["block_n"] == 256 and cfg["split_k"] == 1
+    gen = torch.Generator().manual_seed(21)
+    mask = torch.rand(M, generator=gen) < 0.45
+    w = wl.make_ffn("t", M, d, h, mask, seed=22, w_std=0.03)
+    dw = w.to(dev)
+    out = MaskedFFN.apply(*dw.op_args())
+    x = dw.x.float()
+    ref = torch.empty(M, d, device=dev, dtype=torch.float32)
+    for sel, (k1, k2, k3) in ((dw.mask, ("w1", "w2", "w3")), (~dw.mask, ("u1", "u2", "u3"))):
+        t1 = x[sel] @ dw.W[k1].float().T
+        t3 = x[sel] @ dw.W[k3].float().T
+        hmid = (t1 * torch.sigmoid(t1) * t3).to(torch.bfloat16).float()
+        ref[sel] = hmid @ dw.W[k2].float().T
+    assert_close(out, ref.double().cpu(), "split tail")
+    # twice the same call: the reduce order is fixed
+    assert torch.equal(out, MaskedFFN.apply(*dw.op_args()))
 
 
 def test_linear_fullsize_scaling_is_exact(dev):
