@@ -182,6 +182,14 @@ RoutedPlan linear_plan(int64_t M, int64_t K, int64_t N) {
   if (p.splits == 1) p.tile = routed_tile(M, N, false);
   return p;
 }
+// fp32 partials of the tiled MaskedLinear forward: split-K for the whole GEMM, or the split tail of
+// the 256x256 tile.
+size_t linear_partial_bytes(int64_t M, int64_t K, int64_t N) {
+  const RoutedPlan p = linear_plan(M, K, N);
+  if (p.splits > 1) return ws_align((size_t)p.splits * M * N * 4);
+  if (p.tile == TILE_256x256_W8 && K % 64 == 0) return ws_align((size_t)kTailSlots * 256 * 256 * 4);
+  return 0;
+}
 int down_tile(int64_t M, int64_t d, int64_t h) { return down_plan(M, d, h).tile; }
 int tiled_down_splits(int64_t M, int64_t d, int64_t h) {
   return use_stream_path(M, d, h) ? 1 : down_plan(M, d, h).splits;
@@ -221,8 +229,11 @@ size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
   switch (op) {
     case FFNK_OP_LINEAR_FWD: {
       // perm + counts + the fp32 split-K partials where the GEMM (or the streamed projection) is split
-      const int splits = linear_stream_kind(M, K, N) ? linear_stream_splits(M, K, N) : linear_plan(M, K, N).splits;
-      return route_ws_bytes(M) + (splits > 1 ? ws_align((size_t)splits * M * N * 4) : 0);
+      if (linear_stream_kind(M, K, N)) {
+        const int splits = linear_stream_splits(M, K, N);
+        return route_ws_bytes(M) + (splits > 1 ? ws_align((size_t)splits * M * N * 4) : 0);
+      }
+      return route_ws_bytes(M) + linear_partial_bytes(M, K, N);
     }
     case FFNK_OP_FFN_FWD:
       // perm + counts + the [M, h] bf16 intermediate in routed order (N = h) + the fp32 split-K
@@ -397,6 +408,8 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
   if (plan.splits > 1) {
     g.splits = plan.splits;
     g.P = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + r.bytes);
+  } else if (direct && plan.tile == TILE_256x256_W8) {
+    g.P_tail = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + r.bytes);
   }
   FFNK_HIP(launch_linear_gemm(plan.tile, direct, g, stream), "linear GEMM");
   if (plan.splits > 1)

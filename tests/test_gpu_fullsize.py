@@ -120,6 +120,21 @@ def test_ffn_split_tail_of_the_down_projection(dev):
     assert torch.equal(out, MaskedFFN.apply(*dw.op_args()))
 
 
+def test_linear_split_tail(dev):
+    """MaskedLinear forward on the 256x256 tile with a remainder round that is cut into K ranges."""
+    note("linear split tail M=8500 K=1024 N=4096")
+    M, K, N = 8500, 1024, 4096
+    cfg = _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, N)
+    assert cfg["block_m"] == 256 and cfg["block_n"] == 256 and cfg["split_k"] == 1
+    gen = torch.Generator().manual_seed(31)
+    mask = torch.rand(M, generator=gen) < 0.55
+    w = wl.make_linear("t", M, K, N, mask, seed=32).to(dev)
+    y = MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, w.mask)
+    ref = torch.where(w.mask[:, None], w.x.float() @ w.Wv.float().T, w.x.float() @ w.Wt.float().T)
+    assert_close(y, ref.double().cpu(), "linear split tail")
+    assert torch.equal(y, MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, w.mask))
+
+
 def test_linear_fullsize_scaling_is_exact(dev):
     """y(2x) == 2 y(x) bit for bit (power-of-two scaling commutes with every rounding)."""
     note("cfg1/cfg3-size linear scaling")
