@@ -254,15 +254,23 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
   zero_acc<Cfg>(acc);
   const int nk = k_len / kBK;
 
-  auto issue = [&](int stage, int kt) {
+  auto issue_a = [&](int stage, int kt) {
     uint8_t* st = lds + stage * STAGE;
     const int kb = kt * kRowBytes;
 #pragma unroll
     for (int j = 0; j < NJA; ++j)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[j], FFNK_LDS_PTR(st + (j * NWAVES + wave) * 1024), 16, offA[j], kb, 0, 0);
+  };
+  auto issue_b = [&](int stage, int kt) {
+    uint8_t* st = lds + stage * STAGE;
+    const int kb = kt * kRowBytes;
 #pragma unroll
     for (int j = 0; j < NJB; ++j)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[j], FFNK_LDS_PTR(st + A_BYTES + (j * NWAVES + wave) * 1024), 16, offB[j], kb, 0, 0);
+  };
+  auto issue = [&](int stage, int kt) {
+    issue_a(stage, kt);
+    issue_b(stage, kt);
   };
   bf16x8_t fa[2][TM], fb[2][TN];
   auto load_frags = [&](int buf, int stage, int s) {
@@ -282,10 +290,14 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
   };
 
-  issue(0, 0);
+  // Head of the tile: the weight panels of the first two slabs go out first - their addresses do not
+  // depend on the routing - so that they fly while the gathered token rows' indices are still loading.
+  issue_b(0, 0);
+  if (nk > 1) issue_b(1, 1);
+  issue_a(0, 0);
   if (nk > 1) {
-    issue(1, 1);
-    dma_wait_barrier<L>();
+    issue_a(1, 1);
+    dma_wait_barrier<NJA>();  // in issue order only the token panel of slab 1 may still be under way
   } else {
     dma_wait_barrier<0>();
   }
