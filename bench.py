@@ -1,7 +1,7 @@
 """Headline benchmark: MaskedFFN forward, routed bf16 TFLOP/s at d=4096, h=14336, M=32768 on one
 MI355X (BASELINE.json's metric, `configs[3]`).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4|cfg2|decode1v|decode1t|decode8|decode32|decode64]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4|cfg2|decode1v|decode1t|decode8|decode32|decode64|prefill1024]
 
 A step is one MaskedFFN.apply over the whole synthetic batch (row partition + up-projection with
 SwiGLU + down-projection), inputs already resident in HBM.  Prints ONE JSON line.
@@ -159,6 +159,9 @@ def main() -> int:
         spec = args.workload[6:] or "64"
         kind = {"v": "visual", "t": "text"}.get(spec[-1], "bernoulli")
         w_cpu = wl.cfg5_ffn_decode(int(spec.rstrip("vt")), kind)
+    elif args.workload.startswith("prefill"):
+        # mid-size batches at the cfg4/cfg5 layer shape (Bernoulli mask): few output tiles, split-K down projection
+        w_cpu = wl.cfg5_ffn_decode(int(args.workload[7:] or "1024"), "bernoulli")
     else:
         raise SystemExit(f"unknown workload {args.workload}")
     w = w_cpu.to(dev)

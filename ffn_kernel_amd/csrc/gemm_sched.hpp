@@ -26,6 +26,9 @@ __host__ __device__ inline TileCoord routed_tile_coord(int L, int n_vis, int M, 
   const int tiles_v = cdiv(n_vis, bm);
   const int tiles_m = tiles_v + cdiv(M - n_vis, bm);
   const int tiles_n = cdiv(N, bn);
+  // Up to two groups' worth of M-tiles form a single super-group: a short last group of one or two
+  // M-tiles would stream its weights again with nobody to share them with.
+  if (tiles_m <= 2 * group_m) group_m = tiles_m;
   const int width = group_m * tiles_n;
   const int first_m = (L / width) * group_m;
   const int gsz = group_m < tiles_m - first_m ? group_m : tiles_m - first_m;
