@@ -67,6 +67,23 @@ def test_tile_table_entries():
     assert small["block_m"] * small["block_n"] < 256 * 256  # small problems get small tiles
     tail = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 72, 1024)
     assert tail["direct_lds"] == 0 and tail["block_k"] == 64 and tail["lds_stages"] == 2
+    # few output tiles over a long contraction: the down projection / the linear layer cut K ...
+    for M in (65, 128, 512, 1024, 4096):
+        dn = _lib.tile_config(_lib.OP_FFN_DOWN, M, 4096, 14336)
+        assert dn["path"] == _lib.PATH_MFMA_TILED and dn["split_k"] > 1, (M, dn)
+        assert (14336 // 64) // dn["split_k"] >= 8  # at least eight slabs per range
+        # ... and the workspace holds perm/counts, the [M, h] intermediate and the fp32 partials
+        need = M * 4 + 8 + M * 14336 * 2 + dn["split_k"] * M * 4096 * 4
+        assert _lib.workspace_bytes(_lib.OP_FFN_FWD, M, 4096, 14336) >= need
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 32768, 4096, 14336)["split_k"] == 1
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 2048, 72, 264)["split_k"] == 1      # K % 64 != 0: no split
+    lin = _lib.tile_config(_lib.OP_LINEAR_FWD, 200, 4096, 1024)
+    assert lin["path"] == _lib.PATH_MFMA_TILED and lin["split_k"] > 1
+    assert _lib.workspace_bytes(_lib.OP_LINEAR_FWD, 200, 4096, 1024) >= 200 * 4 + 8 + lin["split_k"] * 200 * 1024 * 4
+    # decode-sized linear calls run on the streaming kernels
+    assert _lib.tile_config(_lib.OP_LINEAR_FWD, 1, 4096, 4096)["path"] == _lib.PATH_STREAM
+    assert _lib.tile_config(_lib.OP_LINEAR_FWD, 64, 4096, 4096)["path"] == _lib.PATH_STREAM
+    assert _lib.tile_config(_lib.OP_LINEAR_FWD, 64, 4096, 4100)["path"] == _lib.PATH_MFMA_TILED  # ragged N
     dw = _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)
     assert dw["split_k"] > 1
     with pytest.raises(ValueError):
