@@ -42,6 +42,20 @@ _SIGNATURES = {
                                     c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,  # dW1 dW3 dU1 dU3
                                     c_void_p, c_void_p, c_int64, c_int64,            # dW2 dU2
                                     c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "ffnk_masked_ffn_can_save": (c_int, [c_int64, c_int64, c_int64]),
+    "ffnk_masked_ffn_fwd_save": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                         c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64,
+                                         c_void_p, c_int64,                          # pre
+                                         c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "ffnk_masked_ffn_bwd_saved": (c_int, [c_void_p, c_int64, c_void_p, c_int64,
+                                          c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                          c_void_p, c_void_p, c_int64, c_int64,
+                                          c_void_p,
+                                          c_void_p, c_int64,                         # pre
+                                          c_void_p, c_int64,
+                                          c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                          c_void_p, c_void_p, c_int64, c_int64,
+                                          c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -426,11 +426,17 @@ int ffnk_masked_ffn_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t* W
                                 down_stride_n, mask, out, out_stride_m, M, d, h, ws, ws_bytes, stream_, nullptr);
 }
 
-int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, const uint16_t* W3,
-                           const uint16_t* U1, const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n,
-                           const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
-                           const uint8_t* mask, uint16_t* out, int64_t out_stride_m, int64_t M, int64_t d,
-                           int64_t h, void* ws, size_t ws_bytes, void* stream_, void* const* events) {
+}  // extern "C"
+
+namespace {
+
+// Forward shared by the entry points.  pre != NULL: also store the two pre-activations (routed order,
+// [M, 2h], gate | up) for a later ffnk_masked_ffn_bwd_saved; only the LDS-tiled path can do that.
+int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, const uint16_t* W3, const uint16_t* U1,
+                 const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n, const uint16_t* W2, const uint16_t* U2,
+                 int64_t down_stride_k, int64_t down_stride_n, const uint8_t* mask, uint16_t* out, int64_t out_stride_m,
+                 uint16_t* pre, int64_t pre_stride_m, int64_t M, int64_t d, int64_t h, void* ws, size_t ws_bytes,
+                 void* stream_, void* const* events) {
   hipStream_t stream = (hipStream_t)stream_;
   auto mark = [&](int i) -> hipError_t {
     if (events && events[i]) return hipEventRecord((hipEvent_t)events[i], stream);
@@ -457,6 +463,14 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
                     up_stride_k == 1 && up_stride_n % 8 == 0 && up_stride_n >= d && down_stride_k == 1 &&
                     down_stride_n % 8 == 0 && down_stride_n >= h && aligned16(W1) && aligned16(W3) &&
                     aligned16(U1) && aligned16(U3) && aligned16(W2) && aligned16(U2);
+  if (pre != nullptr) {
+    if (!fast || use_stream_path(M, d, h))
+      return fail(FFNK_E_STRIDE, "MaskedFFN forward: pre-activations can only be saved on the LDS-tiled path "
+                                 "(M > 64, fast layout); see ffnk_masked_ffn_can_save");
+    if (pre_stride_m < 2 * h || pre_stride_m % 8 != 0 || !aligned16(pre))
+      return fail(FFNK_E_STRIDE, "pre_stride_m=%lld: need >= 2h, a multiple of 8, and 16-byte aligned rows",
+                  (long long)pre_stride_m);
+  }
   if (!fast) {
     // Token-order intermediate, then the generic routed linear on it.
     GenericUpArgs u;
@@ -514,6 +528,7 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
   up.C = H; up.ldc = ldh;
   up.perm = r.perm; up.counts = r.counts;
   up.M = (int)M; up.N = (int)h; up.K = (int)d;
+  up.C_pre = pre; up.ldc_pre = pre_stride_m;
   FFNK_HIP(launch_up_gemm(routed_tile(M, h, true), direct_ok(d, M, x_stride_m, up_stride_n), up, stream), "up-projection GEMM");
   FFNK_HIP(mark(1), "event record");
   GemmArgs dn;
@@ -536,6 +551,34 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
     FFNK_HIP(launch_routed_reduce(dn.P, dn_splits, (int)M, (int)d, r.perm, out, out_stride_m, stream), "down-projection reduce");
   FFNK_HIP(mark(2), "event record");
   return FFNK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, const uint16_t* W3,
+                           const uint16_t* U1, const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n,
+                           const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
+                           const uint8_t* mask, uint16_t* out, int64_t out_stride_m, int64_t M, int64_t d,
+                           int64_t h, void* ws, size_t ws_bytes, void* stream_, void* const* events) {
+  return ffn_fwd_impl(x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k, down_stride_n, mask,
+                      out, out_stride_m, nullptr, 0, M, d, h, ws, ws_bytes, stream_, events);
+}
+
+int ffnk_masked_ffn_can_save(int64_t M, int64_t d, int64_t h) {
+  return (M > 0 && d > 0 && h > 0 && d % 8 == 0 && h % 8 == 0 && !use_stream_path(M, d, h)) ? 1 : 0;
+}
+
+int ffnk_masked_ffn_fwd_save(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, const uint16_t* W3,
+                             const uint16_t* U1, const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n,
+                             const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
+                             const uint8_t* mask, uint16_t* out, int64_t out_stride_m, uint16_t* pre,
+                             int64_t pre_stride_m, int64_t M, int64_t d, int64_t h, void* ws, size_t ws_bytes,
+                             void* stream_) {
+  if (!pre) return fail(FFNK_E_NULL, "pre is NULL");
+  return ffn_fwd_impl(x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k, down_stride_n, mask,
+                      out, out_stride_m, pre, pre_stride_m, M, d, h, ws, ws_bytes, stream_, nullptr);
 }
 
 int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,
@@ -613,15 +656,23 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   return FFNK_OK;
 }
 
-int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,
-                        const uint16_t* W1, const uint16_t* W3, const uint16_t* U1, const uint16_t* U3,
-                        int64_t up_stride_k, int64_t up_stride_n, const uint16_t* W2, const uint16_t* U2,
-                        int64_t down_stride_k, int64_t down_stride_n, const uint8_t* mask, uint16_t* dx,
-                        int64_t dx_stride_m, uint16_t* dW1, uint16_t* dW3, uint16_t* dU1, uint16_t* dU3,
-                        int64_t dup_stride_k, int64_t dup_stride_n, uint16_t* dW2, uint16_t* dU2,
-                        int64_t ddown_stride_k, int64_t ddown_stride_n, int64_t M, int64_t d, int64_t h, void* ws,
-                        size_t ws_bytes, void* stream_) {
+}  // extern "C"
+
+namespace {
+
+// Backward shared by the entry points.  pre != NULL: the pre-activations a forward saved
+// (ffnk_masked_ffn_fwd_save, same mask), read-only; NULL: recompute them with two routed GEMMs.
+int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m, const uint16_t* W1,
+                 const uint16_t* W3, const uint16_t* U1, const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n,
+                 const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
+                 const uint8_t* mask, const uint16_t* pre, int64_t pre_stride_m, uint16_t* dx, int64_t dx_stride_m,
+                 uint16_t* dW1, uint16_t* dW3, uint16_t* dU1, uint16_t* dU3, int64_t dup_stride_k, int64_t dup_stride_n,
+                 uint16_t* dW2, uint16_t* dU2, int64_t ddown_stride_k, int64_t ddown_stride_n, int64_t M, int64_t d,
+                 int64_t h, void* ws, size_t ws_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
+  if (pre != nullptr && (pre_stride_m < 2 * h || pre_stride_m % 8 != 0 || !aligned16(pre)))
+    return fail(FFNK_E_STRIDE, "pre_stride_m=%lld: need >= 2h, a multiple of 8, and 16-byte aligned rows",
+                (long long)pre_stride_m);
   if (int e = check_extents(M, d, h)) return e;
   if (d == 0 || h == 0) return fail(FFNK_E_SHAPE, "MaskedFFN backward needs d > 0 and h > 0");
   if (!W1 || !W3 || !U1 || !U3 || !W2 || !U2 || !dW1 || !dW3 || !dU1 || !dU3 || !dW2 || !dU2)
@@ -654,10 +705,12 @@ int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x
   a.ldc = ld13; a.perm = r.perm; a.counts = r.counts;
   a.M = (int)M; a.N = (int)h; a.K = (int)d;
   const bool up_direct = direct_ok(d, M, x_stride_m, up_stride_n);
-  a.B0[0] = W1; a.B0[1] = U1; a.C = T13;
-  FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), up_direct, a, stream), "t1 GEMM");
-  a.B0[0] = W3; a.B0[1] = U3; a.C = T13 + h;
-  FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), up_direct, a, stream), "t3 GEMM");
+  if (pre == nullptr) {
+    a.B0[0] = W1; a.B0[1] = U1; a.C = T13;
+    FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), up_direct, a, stream), "t1 GEMM");
+    a.B0[0] = W3; a.B0[1] = U3; a.C = T13 + h;
+    FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), up_direct, a, stream), "t3 GEMM");
+  }
 
   // ---- dh = gather(g) @ A2^T: contraction over d needs the down weights as [h, d] rows ----
   const uint16_t* w2t[2] = {W2, U2};
@@ -674,7 +727,8 @@ int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x
   FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), direct_ok(d, M, g_stride_m, ld2), a, stream), "dh GEMM");
 
   // ---- elementwise: T13 <- (dt1 | dt3), DH <- the SwiGLU intermediate ----
-  FFNK_HIP(launch_swiglu_bwd(T13, ld13, DH, h, (int)M, (int)h, stream), "SwiGLU backward pass");
+  FFNK_HIP(launch_swiglu_bwd(pre ? pre : T13, pre ? pre_stride_m : ld13, T13, ld13, DH, h, (int)M, (int)h, stream),
+           "SwiGLU backward pass");
 
   // ---- dx = (dt1 | dt3) @ (A1^T | A3^T)^T: one GEMM over the concatenated contraction of length 2h ----
   uint16_t* w13[2] = {reinterpret_cast<uint16_t*>(wsb + p.off_w13t),
@@ -735,6 +789,37 @@ int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x
   if (int e = weight_grad(p.up, D1T, XT, dW1, dU1, dup_stride_k, dup_stride_n)) return e;
   if (int e = weight_grad(p.up, D3T, XT, dW3, dU3, dup_stride_k, dup_stride_n)) return e;
   return FFNK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,
+                        const uint16_t* W1, const uint16_t* W3, const uint16_t* U1, const uint16_t* U3,
+                        int64_t up_stride_k, int64_t up_stride_n, const uint16_t* W2, const uint16_t* U2,
+                        int64_t down_stride_k, int64_t down_stride_n, const uint8_t* mask, uint16_t* dx,
+                        int64_t dx_stride_m, uint16_t* dW1, uint16_t* dW3, uint16_t* dU1, uint16_t* dU3,
+                        int64_t dup_stride_k, int64_t dup_stride_n, uint16_t* dW2, uint16_t* dU2,
+                        int64_t ddown_stride_k, int64_t ddown_stride_n, int64_t M, int64_t d, int64_t h, void* ws,
+                        size_t ws_bytes, void* stream_) {
+  return ffn_bwd_impl(g, g_stride_m, x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k,
+                      down_stride_n, mask, nullptr, 0, dx, dx_stride_m, dW1, dW3, dU1, dU3, dup_stride_k, dup_stride_n,
+                      dW2, dU2, ddown_stride_k, ddown_stride_n, M, d, h, ws, ws_bytes, stream_);
+}
+
+int ffnk_masked_ffn_bwd_saved(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,
+                              const uint16_t* W1, const uint16_t* W3, const uint16_t* U1, const uint16_t* U3,
+                              int64_t up_stride_k, int64_t up_stride_n, const uint16_t* W2, const uint16_t* U2,
+                              int64_t down_stride_k, int64_t down_stride_n, const uint8_t* mask, const uint16_t* pre,
+                              int64_t pre_stride_m, uint16_t* dx, int64_t dx_stride_m, uint16_t* dW1, uint16_t* dW3,
+                              uint16_t* dU1, uint16_t* dU3, int64_t dup_stride_k, int64_t dup_stride_n, uint16_t* dW2,
+                              uint16_t* dU2, int64_t ddown_stride_k, int64_t ddown_stride_n, int64_t M, int64_t d,
+                              int64_t h, void* ws, size_t ws_bytes, void* stream_) {
+  if (M > 0 && !pre) return fail(FFNK_E_NULL, "pre is NULL");
+  return ffn_bwd_impl(g, g_stride_m, x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k,
+                      down_stride_n, mask, pre, pre_stride_m, dx, dx_stride_m, dW1, dW3, dU1, dU3, dup_stride_k,
+                      dup_stride_n, dW2, dU2, ddown_stride_k, ddown_stride_n, M, d, h, ws, ws_bytes, stream_);
 }
 
 }  // extern "C"

@@ -12,6 +12,11 @@ struct GemmArgs {
   int64_t ldb;
   uint16_t* C;           // [*, N] rows
   int64_t ldc;
+  // SwiGLU kernels only, optional: the two pre-activations, bf16, rows like C (routed order):
+  // C_pre[row, n] = A B0^T, C_pre[row, N + n] = A B1^T.  Saved by a training forward so that the
+  // backward need not recompute them.  NULL: not stored.
+  uint16_t* C_pre = nullptr;
+  int64_t ldc_pre = 0;
   const int32_t* perm;   // routed position -> token row
   const int32_t* counts; // counts[0] = visual rows (device memory)
   int M, N, K;           // N = output columns

@@ -386,6 +386,24 @@ __device__ __forceinline__ void routed_epilogue(const GemmArgs& g, f32x16_t (&ac
           for (int e = 0; e < 4; ++e)
             if (n + e < g.N) crow[n + e] = f2bf(o[e]);
         }
+        if (Cfg::DUAL && g.C_pre != nullptr) {  // uniform over the launch
+          uint16_t* prow = g.C_pre + dst * g.ldc_pre + n;
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const f32x16_t& t = acc[i][j + half * TN_OUT];
+            uint16_t* pp = prow + (int64_t)half * g.N;
+            if (n + 3 < g.N && ((reinterpret_cast<uintptr_t>(pp) & 7) == 0)) {
+              uint2 v2;
+              v2.x = pack2bf(t[4 * q4], t[4 * q4 + 1]);
+              v2.y = pack2bf(t[4 * q4 + 2], t[4 * q4 + 3]);
+              *reinterpret_cast<uint2*>(pp) = v2;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (n + e < g.N) pp[e] = f2bf(t[4 * q4 + e]);
+            }
+          }
+        }
       }
     }
   }

@@ -48,11 +48,13 @@ hipError_t launch_gather_transpose2(const uint16_t* src0, int64_t ld0, int cols0
                                     bool routed0 = false, bool routed1 = false);
 // routedN: source N's rows are already in routed order (row p instead of row perm[p]).
 
-// SwiGLU backward, elementwise and in place over routed-order rows (MaskedFFN backward):
-//   t1 = T13[p, j], t3 = T13[p, h + j], dh = DH[p, j]
+// SwiGLU backward, elementwise over routed-order rows (MaskedFFN backward):
+//   t1 = pre[p, j], t3 = pre[p, h + j], dh = DH[p, j]
 //   T13[p, j] <- dh * t3 * silu'(t1),  T13[p, h + j] <- dh * silu(t1),  DH[p, j] <- silu(t1) * t3
-// T13: [M, 2h] row stride ld13; DH: [M, h] row stride ldh; h % 8 == 0.
-hipError_t launch_swiglu_bwd(uint16_t* T13, int64_t ld13, uint16_t* DH, int64_t ldh, int M, int h, hipStream_t stream);
+// pre, T13: [M, 2h] with row strides ld_pre, ld13 (pre may be T13: in place); DH: [M, h] row stride ldh;
+// h % 8 == 0.
+hipError_t launch_swiglu_bwd(const uint16_t* pre, int64_t ld_pre, uint16_t* T13, int64_t ld13, uint16_t* DH, int64_t ldh,
+                             int M, int h, hipStream_t stream);
 // out_g[r * sr + c * sc] = bf16(sum_s P[g][s][r][c]) for g in {0, 1}.
 hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint16_t* out0, uint16_t* out1,
                                 int64_t sr, int64_t sc, hipStream_t stream);

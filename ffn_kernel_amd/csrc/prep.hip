@@ -156,18 +156,19 @@ hipError_t launch_gather_transpose2(const uint16_t* src0, int64_t ld0, int cols0
 // SwiGLU backward in place (see launch.hpp); 8 columns per thread, fp32 maths, bf16 storage.  The
 // derivative is the textbook one, silu'(t) = s + t s (1 - s) with s = sigmoid(t) (the reference's
 // README.md:159-172 sketches this pass; its derivative term there is not this one and is not used).
-__global__ __launch_bounds__(256) void swiglu_bwd_kernel(uint16_t* __restrict__ T13, int64_t ld13,
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* pre, int64_t ld_pre, uint16_t* T13, int64_t ld13,
                                                          uint16_t* __restrict__ DH, int64_t ldh, int M, int h) {
   const int h8 = h >> 3;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (int64_t)M * h8) return;
   const int p = (int)(idx / h8), j = (int)(idx % h8) * 8;
+  const uint16_t* ps1 = pre + (int64_t)p * ld_pre + j;  // may be T13 itself (in place)
   uint16_t* pt1 = T13 + (int64_t)p * ld13 + j;
   uint16_t* pt3 = pt1 + h;
   uint16_t* pdh = DH + (int64_t)p * ldh + j;
   uint16_t t1[8], t3[8], dh[8];
-  *reinterpret_cast<uint4*>(t1) = *reinterpret_cast<const uint4*>(pt1);
-  *reinterpret_cast<uint4*>(t3) = *reinterpret_cast<const uint4*>(pt3);
+  *reinterpret_cast<uint4*>(t1) = *reinterpret_cast<const uint4*>(ps1);
+  *reinterpret_cast<uint4*>(t3) = *reinterpret_cast<const uint4*>(ps1 + h);
   *reinterpret_cast<uint4*>(dh) = *reinterpret_cast<const uint4*>(pdh);
   uint16_t o1[8], o3[8], oh[8];
 #pragma unroll
@@ -184,11 +185,13 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(uint16_t* __restrict__ 
   *reinterpret_cast<uint4*>(pdh) = *reinterpret_cast<const uint4*>(oh);
 }
 
-hipError_t launch_swiglu_bwd(uint16_t* T13, int64_t ld13, uint16_t* DH, int64_t ldh, int M, int h, hipStream_t stream) {
+hipError_t launch_swiglu_bwd(const uint16_t* pre, int64_t ld_pre, uint16_t* T13, int64_t ld13, uint16_t* DH, int64_t ldh,
+                             int M, int h, hipStream_t stream) {
   if (M <= 0 || h <= 0) return hipSuccess;
-  if (h % 8 != 0 || ld13 % 8 != 0 || ldh % 8 != 0) return hipErrorInvalidValue;
+  if (h % 8 != 0 || ld13 % 8 != 0 || ldh % 8 != 0 || ld_pre % 8 != 0) return hipErrorInvalidValue;
   const int64_t n = (int64_t)M * (h / 8);
-  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3((unsigned)cdiv64(n, 256)), dim3(256), 0, stream, T13, ld13, DH, ldh, M, h);
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3((unsigned)cdiv64(n, 256)), dim3(256), 0, stream, pre, ld_pre, T13, ld13, DH,
+                     ldh, M, h);
   return hipGetLastError();
 }
 

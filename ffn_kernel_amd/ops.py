@@ -148,9 +148,13 @@ def masked_linear_backward(grad: torch.Tensor, a: torch.Tensor, b1: torch.Tensor
     return da, db1, db2
 
 
-def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask) -> torch.Tensor:
+def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre: bool = False):
     """SwiGLU FFN routed by mask.  Replaces _bf16_ffn_forward + _bf16_linear_forward
-    (ops.py:30-32, ffn.py:527-560)."""
+    (ops.py:30-32, ffn.py:527-560).
+
+    save_pre: also return the pre-activations [M, 2h] (routed order, gate | up) for
+    masked_ffn_backward(..., pre=...), or None where the shape runs on a path that cannot keep them
+    (decode sizes, d or h not a multiple of 8); the return value is then the pair (out, pre)."""
     _require_cuda_bf16("a", a, 2)
     for name, w in (("w1", w1), ("w2", w2), ("w3", w3), ("u1", u1), ("u2", u2), ("u3", u3)):
         _require_cuda_bf16(name, w, 2)
@@ -180,24 +184,33 @@ def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask) -> torch.Tensor:
     dsk, dsn = _wstrides(downs[0])
     out = torch.empty((M, d), device=dev, dtype=torch.bfloat16)
     if M == 0 or d == 0:
-        return out
+        return (out, None) if save_pre else out
     lib = _lib.load()
+    pre = None
+    if save_pre and h > 0 and lib.ffnk_masked_ffn_can_save(M, d, h) and usk == 1 and dsk == 1:
+        pre = torch.empty((M, 2 * h), device=dev, dtype=torch.bfloat16)
     with torch.cuda.device(dev):
         ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_FWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
-        rc = lib.ffnk_masked_ffn_fwd(a.data_ptr(), a.stride(0) if M > 1 else max(d, 1), ups[0].data_ptr(),
-                                     ups[1].data_ptr(), ups[2].data_ptr(), ups[3].data_ptr(), usk, usn,
-                                     downs[0].data_ptr(), downs[1].data_ptr(), dsk, dsn, mask.data_ptr(),
-                                     out.data_ptr(), d, M, d, h, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+        head = (a.data_ptr(), a.stride(0) if M > 1 else max(d, 1), ups[0].data_ptr(), ups[1].data_ptr(),
+                ups[2].data_ptr(), ups[3].data_ptr(), usk, usn, downs[0].data_ptr(), downs[1].data_ptr(), dsk, dsn,
+                mask.data_ptr(), out.data_ptr(), d)
+        tail = (M, d, h, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+        if pre is None:
+            rc = lib.ffnk_masked_ffn_fwd(*head, *tail)
+        else:
+            rc = lib.ffnk_masked_ffn_fwd_save(*head, pre.data_ptr(), 2 * h, *tail)
     _lib.check(rc, "ffnk_masked_ffn_fwd")
-    return out
+    return (out, pre) if save_pre else out
 
 
-def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask):
+def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None):
     """(da, dw1, dw2, dw3, du1, du2, du3) of MaskedFFN.  The reference stops at NotImplementedError
     here (ops.py:34-38); the decomposition follows its README sketch (README.md:159-172): routed
     GEMMs around one elementwise SwiGLU-gradient pass.  Weight gradients keep the strides of the
-    weight views they belong to, as the linear backward's do."""
+    weight views they belong to, as the linear backward's do.  pre: the pre-activations that
+    masked_ffn_forward(..., save_pre=True) returned for the same inputs (read-only); None: they are
+    recomputed."""
     _require_cuda_bf16("grad", grad, 2)
     _require_cuda_bf16("a", a, 2)
     for name, w in (("w1", w1), ("w2", w2), ("w3", w3), ("u1", u1), ("u2", u2), ("u3", u3)):
@@ -235,13 +248,18 @@ def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask):
     with torch.cuda.device(dev):
         ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
-        rc = lib.ffnk_masked_ffn_bwd(grad.data_ptr(), grad.stride(0) if M > 1 else d, a.data_ptr(),
-                                     a.stride(0) if M > 1 else d, ups[0].data_ptr(), ups[1].data_ptr(),
-                                     ups[2].data_ptr(), ups[3].data_ptr(), usk, usn, downs[0].data_ptr(),
-                                     downs[1].data_ptr(), dsk, dsn, mask.data_ptr(), da.data_ptr(), d,
-                                     dups[0].data_ptr(), dups[1].data_ptr(), dups[2].data_ptr(), dups[3].data_ptr(),
-                                     gusk, gusn, ddowns[0].data_ptr(), ddowns[1].data_ptr(), gdsk, gdsn, M, d, h,
-                                     ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+        head = (grad.data_ptr(), grad.stride(0) if M > 1 else d, a.data_ptr(), a.stride(0) if M > 1 else d,
+                ups[0].data_ptr(), ups[1].data_ptr(), ups[2].data_ptr(), ups[3].data_ptr(), usk, usn,
+                downs[0].data_ptr(), downs[1].data_ptr(), dsk, dsn, mask.data_ptr())
+        tail = (da.data_ptr(), d, dups[0].data_ptr(), dups[1].data_ptr(), dups[2].data_ptr(), dups[3].data_ptr(),
+                gusk, gusn, ddowns[0].data_ptr(), ddowns[1].data_ptr(), gdsk, gdsn, M, d, h, ws.data_ptr(), ws.numel(),
+                _stream_ptr(dev))
+        if pre is None:
+            rc = lib.ffnk_masked_ffn_bwd(*head, *tail)
+        else:
+            if pre.shape != (M, 2 * h) or pre.dtype != torch.bfloat16 or pre.device != dev or pre.stride(1) != 1:
+                raise ValueError(f"pre must be a bf16 [{M}, {2 * h}] tensor on {dev} with contiguous rows")
+            rc = lib.ffnk_masked_ffn_bwd_saved(*head, pre.data_ptr(), pre.stride(0) if M > 1 else 2 * h, *tail)
     _lib.check(rc, "ffnk_masked_ffn_bwd")
     dw1, dw3, du1, du3 = dups
     dw2, du2 = ddowns
@@ -269,18 +287,29 @@ class MaskedLinear(Function):
 
 class MaskedFFN(Function):
     """Routed SwiGLU FFN (reference: ops.py:27-38).  The backward, which the reference leaves at
-    NotImplementedError, recomputes the pre-activations from the saved inputs."""
+    NotImplementedError, uses the pre-activations that a forward with gradients requested keeps
+    ([M, 2h] bf16; as the reference's unfinished training forward does, ffn.py:116-221), and
+    recomputes them from the saved inputs where the forward could not keep them (decode sizes)."""
 
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, a, w1, w2, w3, u1, u2, u3, mask):
-        ctx.save_for_backward(a, mask)
         ctx.weights = (w1, w2, w3, u1, u2, u3)
-        return masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask)
+        if any(ctx.needs_input_grad):
+            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre=True)
+        else:
+            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask), None
+        ctx.has_pre = pre is not None
+        if pre is None:
+            ctx.save_for_backward(a, mask)
+        else:
+            ctx.save_for_backward(a, mask, pre)
+        return out
 
     @staticmethod
     @once_differentiable
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad):
-        a, mask = ctx.saved_tensors
-        return (*masked_ffn_backward(grad, a, *ctx.weights, mask), None)
+        a, mask = ctx.saved_tensors[:2]
+        pre = ctx.saved_tensors[2] if ctx.has_pre else None
+        return (*masked_ffn_backward(grad, a, *ctx.weights, mask, pre=pre), None)

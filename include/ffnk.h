@@ -218,6 +218,52 @@ FFNK_API int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m,
                         int64_t M, int64_t d, int64_t h,
                         void* ws, size_t ws_bytes, void* stream);
 
+/*
+ * Training forward / backward pair that keeps the pre-activations instead of recomputing them.
+ * No counterpart in the live reference (its forward keeps nothing; the dead work-in-progress forward
+ * of ffn_kernel/ffn.py:116-221 stores t1 and t3 for the same purpose).
+ *
+ * ffnk_masked_ffn_fwd_save is ffnk_masked_ffn_fwd and additionally writes pre: [M, 2h] bf16, row
+ * stride pre_stride_m (>= 2h, multiple of 8, rows 16-byte aligned), rows in ROUTED order (visual
+ * rows first, each group ascending), columns [0, h) = t1 = x A1, [h, 2h) = t3 = x A3, rounded to
+ * bf16 from the fp32 accumulators - what the recomputing backward would produce.  Only the LDS-tiled
+ * path can do it: ffnk_masked_ffn_can_save(M, d, h) says whether this shape qualifies (M > 64, d and h
+ * multiples of 8); the fast layout of ffnk_masked_ffn_fwd is required on top.  FFNK_E_STRIDE otherwise.
+ *
+ * ffnk_masked_ffn_bwd_saved is ffnk_masked_ffn_bwd with those pre-activations (same mask), read-only:
+ * it skips the two recompute GEMMs (a quarter of the backward's GEMM work).
+ */
+FFNK_API int ffnk_masked_ffn_can_save(int64_t M, int64_t d, int64_t h);
+
+FFNK_API int ffnk_masked_ffn_fwd_save(const uint16_t* x, int64_t x_stride_m,
+                             const uint16_t* W1, const uint16_t* W3,
+                             const uint16_t* U1, const uint16_t* U3,
+                             int64_t up_stride_k, int64_t up_stride_n,
+                             const uint16_t* W2, const uint16_t* U2,
+                             int64_t down_stride_k, int64_t down_stride_n,
+                             const uint8_t* mask,
+                             uint16_t* out, int64_t out_stride_m,
+                             uint16_t* pre, int64_t pre_stride_m,
+                             int64_t M, int64_t d, int64_t h,
+                             void* ws, size_t ws_bytes, void* stream);
+
+FFNK_API int ffnk_masked_ffn_bwd_saved(const uint16_t* g, int64_t g_stride_m,
+                              const uint16_t* x, int64_t x_stride_m,
+                              const uint16_t* W1, const uint16_t* W3,
+                              const uint16_t* U1, const uint16_t* U3,
+                              int64_t up_stride_k, int64_t up_stride_n,
+                              const uint16_t* W2, const uint16_t* U2,
+                              int64_t down_stride_k, int64_t down_stride_n,
+                              const uint8_t* mask,
+                              const uint16_t* pre, int64_t pre_stride_m,
+                              uint16_t* dx, int64_t dx_stride_m,
+                              uint16_t* dW1, uint16_t* dW3, uint16_t* dU1, uint16_t* dU3,
+                              int64_t dup_stride_k, int64_t dup_stride_n,
+                              uint16_t* dW2, uint16_t* dU2,
+                              int64_t ddown_stride_k, int64_t ddown_stride_n,
+                              int64_t M, int64_t d, int64_t h,
+                              void* ws, size_t ws_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -432,6 +432,49 @@ def test_ffn_bwd_vs_oracle(dev, M, d, h, p):
         assert (Wp[k].grad == 0).all()
 
 
+@pytest.mark.parametrize("M,d,h,p", [(300, 256, 512, 0.5), (1000, 512, 384, 0.3), (777, 128, 320, 1.0), (4500, 1024, 1024, 0.6)])
+def test_ffn_saved_pre_activations(dev, M, d, h, p):
+    """A forward that keeps the pre-activations returns the same output, pre-activations that match the
+    oracle's t1 | t3 in routed order, and a backward from them that equals the recomputing backward
+    bit for bit (both take the same GEMM sums through the same bf16 rounding)."""
+    note(f"ffn saved pre-activations M={M} d={d} h={h} p={p}")
+    from ffn_kernel_amd.ops import masked_ffn_backward, masked_ffn_forward
+    gen = torch.Generator().manual_seed(M + 17)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_ffn("t", M, d, h, mask, seed=M + 1, w_std=0.05)
+    dw = w.to(dev)
+    args = (dw.x, dw.W["w1"].T, dw.W["w2"].T, dw.W["w3"].T, dw.W["u1"].T, dw.W["u2"].T, dw.W["u3"].T, dw.mask)
+    out_plain = masked_ffn_forward(*args)
+    out, pre = masked_ffn_forward(*args, save_pre=True)
+    assert pre is not None and pre.shape == (M, 2 * h) and pre.dtype == torch.bfloat16
+    assert torch.equal(out, out_plain)
+    perm, _ = om.stable_partition(mask.numpy())
+    xr = w.x.double()[torch.from_numpy(perm).long()]
+    mr = mask[torch.from_numpy(perm).long()]
+    t1 = torch.where(mr[:, None], xr @ w.W["w1"].double().T, xr @ w.W["u1"].double().T)
+    t3 = torch.where(mr[:, None], xr @ w.W["w3"].double().T, xr @ w.W["u3"].double().T)
+    assert_close(pre[:, :h], t1, "saved t1")
+    assert_close(pre[:, h:], t3, "saved t3")
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16).to(dev)
+    keep = pre.clone()
+    a = masked_ffn_backward(g, *args)
+    b = masked_ffn_backward(g, *args, pre=pre)
+    assert torch.equal(pre, keep)  # read-only
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)
+
+
+def test_ffn_forward_keeps_nothing_at_decode_sizes(dev):
+    note("ffn save_pre at decode sizes")
+    from ffn_kernel_amd.ops import masked_ffn_forward
+    w = wl.cfg5_ffn_decode(24, "bernoulli", seed=3, d=1024, h=2048).to(dev)
+    out, pre = masked_ffn_forward(*w.op_args(), save_pre=True)
+    assert pre is None and torch.equal(out, masked_ffn_forward(*w.op_args()))
+    x = w.x.clone().requires_grad_(True)
+    MaskedFFN.apply(x, *w.op_args()[1:]).sum().backward()  # recomputing backward
+    assert x.grad is not None and torch.isfinite(x.grad).all()
+
+
 def test_ffn_bwd_is_deterministic_and_validates(dev):
     note("ffn bwd determinism / validation")
     from ffn_kernel_amd.ops import masked_ffn_backward
