@@ -450,6 +450,14 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
       !aligned2(W2) || !aligned2(U2))
     return fail(FFNK_E_ALIGN, "bf16 pointer not 2-byte aligned");
   if (out_stride_m < d) return fail(FFNK_E_STRIDE, "out_stride_m=%lld < d=%lld", (long long)out_stride_m, (long long)d);
+  if (pre != nullptr) {
+    if (!ffnk_masked_ffn_can_save(M, d, h))
+      return fail(FFNK_E_STRIDE, "MaskedFFN forward: pre-activations can only be saved on the LDS-tiled path "
+                                 "(ffnk_masked_ffn_can_save)");
+    if (pre_stride_m < 2 * h || pre_stride_m % 8 != 0 || !aligned16(pre))
+      return fail(FFNK_E_STRIDE, "pre_stride_m=%lld: need >= 2h, a multiple of 8, and 16-byte aligned rows",
+                  (long long)pre_stride_m);
+  }
   const size_t need = ffnk_workspace_bytes(FFNK_OP_FFN_FWD, M, d, h);
   if (ws_bytes < need || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, need);
   if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
@@ -463,14 +471,9 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
                     up_stride_k == 1 && up_stride_n % 8 == 0 && up_stride_n >= d && down_stride_k == 1 &&
                     down_stride_n % 8 == 0 && down_stride_n >= h && aligned16(W1) && aligned16(W3) &&
                     aligned16(U1) && aligned16(U3) && aligned16(W2) && aligned16(U2);
-  if (pre != nullptr) {
-    if (!fast || use_stream_path(M, d, h))
-      return fail(FFNK_E_STRIDE, "MaskedFFN forward: pre-activations can only be saved on the LDS-tiled path "
-                                 "(M > 64, fast layout); see ffnk_masked_ffn_can_save");
-    if (pre_stride_m < 2 * h || pre_stride_m % 8 != 0 || !aligned16(pre))
-      return fail(FFNK_E_STRIDE, "pre_stride_m=%lld: need >= 2h, a multiple of 8, and 16-byte aligned rows",
-                  (long long)pre_stride_m);
-  }
+  if (pre != nullptr && !fast)
+    return fail(FFNK_E_STRIDE, "MaskedFFN forward: saving the pre-activations needs the fast layout (16-byte aligned, "
+                               "K-contiguous operands)");
   if (!fast) {
     // Token-order intermediate, then the generic routed linear on it.
     GenericUpArgs u;

@@ -118,6 +118,30 @@ def test_ffn_backward_entry_rejects_bad_arguments_without_a_gpu():
     assert need >= _lib.workspace_bytes(_lib.OP_FFN_FWD, 8192, 1024, 2048)
 
 
+def test_ffn_save_entries_reject_bad_arguments_without_a_gpu():
+    """The training forward that keeps the pre-activations and the backward that reads them."""
+    lib = _lib.load()
+    P = ctypes.c_void_p
+    one = P(16)
+    assert lib.ffnk_masked_ffn_can_save(4096, 4096, 14336) == 1
+    assert lib.ffnk_masked_ffn_can_save(64, 4096, 14336) == 0   # decode sizes stream the weights
+    assert lib.ffnk_masked_ffn_can_save(300, 36, 20) == 0       # any-stride kernels
+    def fwd(M=128, d=64, h=64, pre=one, pre_stride=128, ws=None, ws_bytes=0):
+        return lib.ffnk_masked_ffn_fwd_save(one, d, one, one, one, one, 1, d, one, one, 1, h, one, one, d, pre, pre_stride,
+                                            M, d, h, ws, ws_bytes, None)
+    assert fwd(pre=None) == -1
+    assert fwd(M=8, d=1024, h=1024, pre_stride=2048) == -3 and b"LDS-tiled" in lib.ffnk_last_error()  # decode size
+    assert fwd(pre_stride=64) == -3                                    # rows shorter than 2h
+    assert fwd() == -5                                                 # passes validation, no workspace
+    def bwd(pre=one, pre_stride=128):
+        return lib.ffnk_masked_ffn_bwd_saved(one, 64, one, 64, one, one, one, one, 1, 64, one, one, 1, 64, one, pre,
+                                             pre_stride, one, 64, one, one, one, one, 1, 64, one, one, 1, 64, 128, 64, 64,
+                                             None, 0, None)
+    assert bwd(pre=None) == -1
+    assert bwd(pre_stride=100) == -3
+    assert bwd() == -5
+
+
 def test_ops_validate_inputs():
     x = torch.zeros(4, 8, dtype=torch.bfloat16)
     w = torch.zeros(8, 8, dtype=torch.bfloat16)
