@@ -48,6 +48,9 @@ inline hipError_t dispatch_tile_with_tail(int tile, const GemmArgs& g, hipStream
   using Big = typename Tiles::T0;
   using Small = typename Tiles::T2;
   if (tile != TILE_256x256_W8 || g.splits > 1 || g.M <= 0 || g.N <= 0) return dispatch_tile<Tiles>(tile, g, stream);
+  // At most one round of big tiles: nothing to split off (every tile would land in the remainder).
+  if ((int64_t)(cdiv(g.M, Tiles::T0::BM) + 1) * cdiv(g.N, Tiles::T0::BN_OUT) <= kCusPerChip)
+    return dispatch_tile<Tiles>(tile, g, stream);
   GemmArgs a = g;
   a.tail_mode = 1;
   if (hipError_t e = launch_routed_gemm<Big>(a, stream)) return e;
