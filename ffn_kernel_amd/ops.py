@@ -8,6 +8,8 @@ Same class names, same positional signatures:
 """
 from __future__ import annotations
 
+import threading
+
 import torch
 from torch.autograd import Function
 from torch.autograd.function import once_differentiable
@@ -266,6 +268,13 @@ def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None):
     return da, dw1, dw2, dw3, du1, du2, du3
 
 
+class _GradMode(threading.local):
+    enabled = True
+
+
+_grad_mode = _GradMode()
+
+
 class MaskedLinear(Function):
     """c = a @ (b1 where mask else b2), forward and backward (reference: ops.py:9-24)."""
 
@@ -291,11 +300,19 @@ class MaskedFFN(Function):
     ([M, 2h] bf16; as the reference's unfinished training forward does, ffn.py:116-221), and
     recomputes them from the saved inputs where the forward could not keep them (decode sizes)."""
 
+    @classmethod
+    def apply(cls, *args, **kwargs):
+        # forward() always runs with gradients switched off and ctx.needs_input_grad does not say whether
+        # the caller is under torch.no_grad(): note it here, so that evaluation does not pay for keeping
+        # the pre-activations
+        _grad_mode.enabled = torch.is_grad_enabled()
+        return super().apply(*args, **kwargs)
+
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, a, w1, w2, w3, u1, u2, u3, mask):
         ctx.weights = (w1, w2, w3, u1, u2, u3)
-        if any(ctx.needs_input_grad):
+        if _grad_mode.enabled and any(ctx.needs_input_grad):
             out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre=True)
         else:
             out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask), None

@@ -641,3 +641,24 @@ def test_ffn_forward_is_graph_capturable(dev, M, d, h):
         eager = MaskedFFN.apply(x_new, *w.op_args()[1:])
         torch.cuda.synchronize()
         assert torch.equal(out_static, eager), rep
+
+
+def test_ffn_forward_keeps_pre_activations_only_when_a_backward_can_follow(dev, monkeypatch):
+    note("ffn save_pre decision")
+    from ffn_kernel_amd import ops
+    seen = []
+    real = ops.masked_ffn_forward
+    def spy(*args, save_pre=False):
+        seen.append(save_pre)
+        return real(*args, save_pre=save_pre)
+    monkeypatch.setattr(ops, "masked_ffn_forward", spy)
+    mask = torch.rand(200, generator=torch.Generator().manual_seed(1)) < 0.5
+    w = wl.make_ffn("t", 200, 128, 256, mask, seed=2, w_std=0.05).to(dev)
+    args = w.op_args()
+    MaskedFFN.apply(*args)                                   # nothing requires grad
+    x = args[0].clone().requires_grad_(True)
+    with torch.no_grad():
+        MaskedFFN.apply(x, *args[1:])                        # evaluation with trainable inputs
+    out = MaskedFFN.apply(x, *args[1:])                      # training
+    out.sum().backward()
+    assert seen == [False, False, True] and x.grad is not None
