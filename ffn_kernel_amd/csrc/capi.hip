@@ -126,6 +126,14 @@ bool direct_ok(int64_t K, int64_t gathered_rows, int64_t lda, int64_t ldb) {
   return 256 * lda * 2 < k4g && 256 * ldb * 2 < k4g;
 }
 
+// The K-major kernels read a weight where the backward finds it: [K, N] rows of the contraction, N
+// contiguous, row stride ldb.  Slabs are addressed with 32-bit byte offsets from their first row.
+bool kmajor_ok(int64_t K, int64_t N, int64_t ldb, const void* w0, const void* w1) {
+  constexpr int64_t k4g = (int64_t)1 << 32;
+  return K > 0 && K % 64 == 0 && N >= 8 && N % 8 == 0 && ldb % 8 == 0 && ldb >= N && aligned16(w0) && aligned16(w1) &&
+         ldb * 128 + 2 * N < k4g;
+}
+
 int g_force_tile = -1;  // tuner override, see ffnk_debug_force_tile
 
 int routed_tile(int64_t M, int64_t n_out, bool dual) {
@@ -624,7 +632,11 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   const uint16_t* wt[2] = {Wv, Wt};
   int64_t ldw = w_stride_k;
   const bool w_direct = w_stride_n == 1 && w_stride_k % 8 == 0 && w_stride_k >= N && aligned16(Wv) && aligned16(Wt);
-  if (!w_direct) {
+  // The forward's layout ([N, K] rows, K contiguous) is K-major for this GEMM: no copy either.
+  const bool w_kmajor = !w_direct && w_stride_k == 1 && kmajor_ok(N, K, w_stride_n, Wv, Wt) && direct_ok(N, M, g_stride_m, 8);
+  if (w_kmajor) {
+    ldw = w_stride_n;
+  } else if (!w_direct) {
     uint16_t* c0 = reinterpret_cast<uint16_t*>(wsb + p.off_wt);
     uint16_t* c1 = reinterpret_cast<uint16_t*>(wsb + p.off_wt + ws_align((size_t)K * N * 2));
     FFNK_HIP(launch_strided_copy2d(Wv, w_stride_k, w_stride_n, c0, N, (int)K, (int)N, stream), "weight transpose");
@@ -637,7 +649,8 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   a.C = dx; a.ldc = dx_stride_m;
   a.perm = r.perm; a.counts = r.counts;
   a.M = (int)M; a.N = (int)K; a.K = (int)N;
-  FFNK_HIP(launch_linear_gemm(routed_tile(M, K, false), direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
+  if (w_kmajor) FFNK_HIP(launch_linear_gemm_kmajor(routed_tile(M, K, false), a, stream), "dx GEMM");
+  else FFNK_HIP(launch_linear_gemm(routed_tile(M, K, false), direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
 
   // ---- dW_g = x_g^T g_g, contraction over the rows of group g ----
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]
@@ -718,7 +731,13 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   // ---- dh = gather(g) @ A2^T: contraction over d needs the down weights as [h, d] rows ----
   const uint16_t* w2t[2] = {W2, U2};
   int64_t ld2 = down_stride_k;
-  if (!(down_stride_n == 1 && down_stride_k % 8 == 0 && down_stride_k >= d && aligned16(W2) && aligned16(U2))) {
+  const bool w2_direct = down_stride_n == 1 && down_stride_k % 8 == 0 && down_stride_k >= d && aligned16(W2) && aligned16(U2);
+  // The forward's layout ([d, h] rows, h contiguous) is K-major for this GEMM: read in place.
+  const bool w2_kmajor = !w2_direct && down_stride_k == 1 && kmajor_ok(d, h, down_stride_n, W2, U2) &&
+                         direct_ok(d, M, g_stride_m, 8);
+  if (w2_kmajor) {
+    ld2 = down_stride_n;
+  } else if (!w2_direct) {
     uint16_t* c0 = reinterpret_cast<uint16_t*>(wsb + p.off_w2t);
     uint16_t* c1 = reinterpret_cast<uint16_t*>(wsb + p.off_w2t + ws_align((size_t)h * d * 2));
     FFNK_HIP(launch_strided_copy2d(W2, down_stride_k, down_stride_n, c0, d, (int)h, (int)d, stream), "weight transpose");
@@ -727,27 +746,38 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   }
   a.A = g; a.lda = g_stride_m; a.B0[0] = w2t[0]; a.B0[1] = w2t[1]; a.ldb = ld2;
   a.C = DH; a.ldc = h;
-  FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), direct_ok(d, M, g_stride_m, ld2), a, stream), "dh GEMM");
+  if (w2_kmajor) FFNK_HIP(launch_gather_gemm_kmajor(routed_tile(M, h, false), a, stream), "dh GEMM");
+  else FFNK_HIP(launch_gather_gemm(routed_tile(M, h, false), direct_ok(d, M, g_stride_m, ld2), a, stream), "dh GEMM");
 
   // ---- elementwise: T13 <- (dt1 | dt3), DH <- the SwiGLU intermediate ----
   FFNK_HIP(launch_swiglu_bwd(pre ? pre : T13, pre ? pre_stride_m : ld13, T13, ld13, DH, h, (int)M, (int)h, stream),
            "SwiGLU backward pass");
 
   // ---- dx = (dt1 | dt3) @ (A1^T | A3^T)^T: one GEMM over the concatenated contraction of length 2h ----
-  uint16_t* w13[2] = {reinterpret_cast<uint16_t*>(wsb + p.off_w13t),
-                      reinterpret_cast<uint16_t*>(wsb + p.off_w13t + ws_align((size_t)d * 2 * h * 2))};
-  FFNK_HIP(launch_strided_copy2d(W1, up_stride_k, up_stride_n, w13[0], ld13, (int)d, (int)h, stream), "weight transpose");
-  FFNK_HIP(launch_strided_copy2d(W3, up_stride_k, up_stride_n, w13[0] + h, ld13, (int)d, (int)h, stream), "weight transpose");
-  FFNK_HIP(launch_strided_copy2d(U1, up_stride_k, up_stride_n, w13[1], ld13, (int)d, (int)h, stream), "weight transpose");
-  FFNK_HIP(launch_strided_copy2d(U3, up_stride_k, up_stride_n, w13[1] + h, ld13, (int)d, (int)h, stream), "weight transpose");
+  // The up-projection weights ([h, d] rows, d contiguous) are K-major for this GEMM: the contraction
+  // runs through the gate weight's rows and on into the up weight's.  Otherwise both are copied
+  // into one [d, 2h] operand per modality.
+  const bool w13_kmajor = h % 64 == 0 && kmajor_ok(2 * h, d, up_stride_n, W1, W3) && aligned16(U1) && aligned16(U3) &&
+                          direct_ok(2 * h, 0, ld13, 8);
   GemmArgs b;
   b.A = T13; b.lda = ld13;
-  b.B0[0] = w13[0]; b.B0[1] = w13[1]; b.B1[0] = b.B1[1] = nullptr; b.ldb = ld13;
+  if (w13_kmajor) {
+    b.B0[0] = W1; b.B0[1] = U1; b.B1[0] = W3; b.B1[1] = U3; b.ldb = up_stride_n;
+    b.k_switch = (int)h;
+  } else {
+    uint16_t* w13[2] = {reinterpret_cast<uint16_t*>(wsb + p.off_w13t),
+                        reinterpret_cast<uint16_t*>(wsb + p.off_w13t + ws_align((size_t)d * 2 * h * 2))};
+    FFNK_HIP(launch_strided_copy2d(W1, up_stride_k, up_stride_n, w13[0], ld13, (int)d, (int)h, stream), "weight transpose");
+    FFNK_HIP(launch_strided_copy2d(W3, up_stride_k, up_stride_n, w13[0] + h, ld13, (int)d, (int)h, stream), "weight transpose");
+    FFNK_HIP(launch_strided_copy2d(U1, up_stride_k, up_stride_n, w13[1], ld13, (int)d, (int)h, stream), "weight transpose");
+    FFNK_HIP(launch_strided_copy2d(U3, up_stride_k, up_stride_n, w13[1] + h, ld13, (int)d, (int)h, stream), "weight transpose");
+    b.B0[0] = w13[0]; b.B0[1] = w13[1]; b.B1[0] = b.B1[1] = nullptr; b.ldb = ld13;
+  }
   b.C = dx; b.ldc = dx_stride_m; b.perm = r.perm; b.counts = r.counts;
   b.M = (int)M; b.N = (int)d; b.K = (int)(2 * h);
   // Few output tiles over a 2h-long contraction: split K like the forward's down projection.  The
   // fp32 partials live where the W2^T copies were (dead since the dh GEMM), if they fit there.
-  const bool dx_direct = direct_ok(2 * h, 0, ld13, ld13);
+  const bool dx_direct = w13_kmajor || direct_ok(2 * h, 0, ld13, ld13);
   RoutedPlan dxp = down_plan(M, d, 2 * h);
   if (!dx_direct || (size_t)dxp.splits * M * d * 4 > 2 * ws_align((size_t)h * d * 2)) {
     dxp.splits = 1;
@@ -756,8 +786,12 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   if (dxp.splits > 1) {
     b.splits = dxp.splits;
     b.P = reinterpret_cast<float*>(wsb + p.off_w2t);
+  } else if (dx_direct && dxp.tile == TILE_256x256_W8 &&
+             (size_t)kTailSlots * 256 * 256 * 4 <= 2 * ws_align((size_t)h * d * 2)) {
+    b.P_tail = reinterpret_cast<float*>(wsb + p.off_w2t);  // split tail of the last, partial round
   }
-  FFNK_HIP(launch_down_gemm(dxp.tile, dx_direct, b, stream), "dx GEMM");
+  if (w13_kmajor) FFNK_HIP(launch_down_gemm_kmajor(dxp.tile, b, stream), "dx GEMM");
+  else FFNK_HIP(launch_down_gemm(dxp.tile, dx_direct, b, stream), "dx GEMM");
   if (dxp.splits > 1)
     FFNK_HIP(launch_routed_reduce(b.P, dxp.splits, (int)M, (int)d, r.perm, dx, dx_stride_m, stream), "dx reduce");
 

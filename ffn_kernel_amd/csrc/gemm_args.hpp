@@ -10,6 +10,11 @@ struct GemmArgs {
   const uint16_t* B0[2]; // per group (0 = visual, 1 = text): [N, K] rows, K contiguous
   const uint16_t* B1[2]; // SwiGLU kernels only: second weight (the "up" projection), same shape
   int64_t ldb;
+  // K-major kernels (weights where the backward finds them): B0[g] is [K, N] rows, N contiguous, row
+  // stride ldb.  With k_switch > 0 (a multiple of 64) the contraction continues in B1[g]: row k of the
+  // operand is B0[g] row k for k < k_switch and B1[g] row k - k_switch after it (two weights that
+  // share the output axis, contracted in one pass).  0: B0 all the way.
+  int k_switch = 0;
   uint16_t* C;           // [*, N] rows
   int64_t ldc;
   // SwiGLU kernels only, optional: the two pre-activations, bf16, rows like C (routed order):

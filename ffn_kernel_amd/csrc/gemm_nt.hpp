@@ -10,6 +10,7 @@
 // otherwise); wavefronts read 16-byte MFMA fragments from an XOR-swizzled LDS layout and issue
 // v_mfma_f32_32x32x16_bf16.
 #pragma once
+#include <type_traits>
 #include "common.hpp"
 #include "gemm_args.hpp"
 #include "gemm_sched.hpp"
@@ -32,8 +33,56 @@ __host__ __device__ constexpr uint32_t lds_swizzle(uint32_t r, uint32_t c) {  //
 
 #define FFNK_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
+// ---------------------------------------------------------------------------------------------
+// K-major weight panels (RoutedGemmCfg::B_KMAJOR).  The backward GEMMs contract over the axis that
+// is the forward's output axis, so they find a weight as [K, N] rows with N contiguous.  A slab of
+// such a panel is 64 rows of BN elements, stored row by row in LDS (again in lane order of the
+// global->LDS loads).  ds_read_b64_tr_b16 turns it into MFMA operands: within a group of 16 lanes,
+// lane j addresses 4 consecutive elements and lane i receives elements i, 16 + i, 32 + i, 48 + i of
+// the 64 the group addressed.  With lanes 4r ... 4r+3 on 16 consecutive columns of row k + r, lane i
+// gets column i of rows k ... k+3; two reads make the 8-element K run of a 32x32x16 operand.
+// Rows are BN * 2 bytes, a multiple of the 256 bytes the banks span, so the four rows of a read are
+// spread by XOR-ing the 64-byte unit index of a row with kmajor_swizzle_key(row).
+// ---------------------------------------------------------------------------------------------
+template <int BN>
+__host__ __device__ constexpr uint32_t kmajor_swizzle_key(uint32_t k) {
+  return BN >= 128 ? (k & 3u) : ((k >> 1) & 1u);  // BN = 64: rows 128 bytes apart, two units each
+}
+
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+
+// The transposing read is written as an asm statement: through its builtin the compiler takes it for
+// a possible LDS store and puts s_waitcnt vmcnt(0) before every one that follows a global->LDS load,
+// which would drain the slab prefetch at each K step.  The compiler therefore does not know that the
+// result arrives later: kmajor_wait_frags() must stand between the reads and the first use.
+template <int OFFSET>
+__device__ __forceinline__ bf16x4_t lds_read_tr16_b64(uint32_t addr) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536, "DS offset field is 16 bits");
+  bf16x4_t r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFFSET));
+  return r;
+}
+// Wait for every outstanding LDS read of the wave; the fragments pass through the statement so that
+// no use of them can be moved above it.
+template <int TN>
+__device__ __forceinline__ void kmajor_wait_frags(bf16x4_t (&lo)[TN], bf16x4_t (&hi)[TN]) {
+  static_assert(TN == 1 || TN == 2 || TN == 4, "weight fragments per K step");
+  if constexpr (TN == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[0]), "+v"(hi[0]));
+  if constexpr (TN == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[0]), "+v"(hi[0]), "+v"(lo[1]), "+v"(hi[1]));
+  if constexpr (TN == 4)
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(lo[0]), "+v"(hi[0]), "+v"(lo[1]), "+v"(hi[1]), "+v"(lo[2]), "+v"(hi[2]), "+v"(lo[3]), "+v"(hi[3]));
+}
+
+struct KMajorB {
+  const uint16_t* w[2] = {nullptr, nullptr};  // slabs [0, kt_switch) of the contraction come from w[0], the rest from w[1]
+  int kt_first = 0;                           // first slab of this workgroup's K range
+  int kt_switch = 0x7fffffff;
+  uint32_t slab_bytes = 0;                    // 64 rows: 64 * ldb * 2
+};
+
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool DUAL_, bool GATHER_A_, bool SCATTER_C_,
-          bool DIRECT_, int GROUP_M_>
+          bool DIRECT_, int GROUP_M_, bool B_KMAJOR_ = false>
 struct RoutedGemmCfg {
   static constexpr int BM = BM_;            // token rows per tile
   static constexpr int BN = BN_;            // B rows held in LDS per tile (DUAL: half gate, half up)
@@ -44,6 +93,9 @@ struct RoutedGemmCfg {
   static constexpr bool SCATTER_C = SCATTER_C_;
   static constexpr bool DIRECT = DIRECT_;   // global->LDS loads bypass registers (needs K % 64 == 0)
   static constexpr int GROUP_M = GROUP_M_;
+  // Weight panels are [K, N] rows with N contiguous (the backward's view of a forward weight) and
+  // are transposed on the way from LDS to the MFMA operand, see KMajorB.
+  static constexpr bool B_KMAJOR = B_KMAJOR_;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int NT = NWAVES * kWave;
   static constexpr int BN_OUT = DUAL ? BN / 2 : BN;        // output columns per tile
@@ -59,6 +111,7 @@ struct RoutedGemmCfg {
   static_assert(NWAVES % 2 == 0, "lane mapping of the slab layout needs an even wave count");
   static_assert((BM / 16) % NWAVES == 0 && (BN / 16) % NWAVES == 0, "panel rows must split evenly over waves");
   static_assert(!DUAL || (BN / 2) % 16 == 0, "gate/up split must fall on a 16-row load group");
+  static_assert(!B_KMAJOR || (DIRECT && !DUAL && BN >= 64 && BN <= 512), "K-major weights: direct path, one weight");
 };
 
 // Accumulator tile b of the wave reads B-panel rows starting here.
@@ -103,6 +156,12 @@ struct TileLanes {
   uint32_t r_in;   // row inside the 8-row group this lane loads
   uint32_t c_log;  // logical 16-byte chunk (0..7) of that row
   uint32_t lr, lh; // MFMA fragment row (0..31) and K half (0..1)
+  // K-major weight panel: a 64-row slab of BN-element rows is moved as 1 KB groups of 64 / (BN / 8)
+  // whole rows; this lane fills physical slot `lane` of its group, which holds logical chunk kb_chunk
+  // of row kb_row of the group.
+  uint32_t kb_row, kb_chunk;
+  static constexpr int KB_CPR = Cfg::BN / 8;    // 16-byte chunks per K-major row
+  static constexpr int KB_RPG = 64 / (KB_CPR > 64 ? 64 : KB_CPR);  // rows per 1 KB group
 
   __device__ __forceinline__ void init() {
     const int tid = threadIdx.x;
@@ -117,7 +176,17 @@ struct TileLanes {
     c_log = (q & 7) ^ r_in;
     lr = lane & 31;
     lh = lane >> 5;
+    kb_row = kb_chunk = 0;
+    if (Cfg::B_KMAJOR) {
+      static_assert(!Cfg::B_KMAJOR || (KB_CPR <= 64 && (KB_RPG == 2 || KB_RPG == 4 || KB_RPG == 8)), "BN of 64, 128 or 256");
+      kb_row = lane / KB_CPR;
+      const uint32_t c_phys = lane % KB_CPR;
+      // kmajor_swizzle_key() of slab row group * KB_RPG + kb_row; the group's parity is the wave's.
+      const uint32_t key = KB_RPG == 2 ? 2 * (wave & 1) + kb_row : KB_RPG == 4 ? kb_row : (kb_row >> 1) & 1;
+      kb_chunk = (((c_phys >> 2) ^ key) << 2) | (c_phys & 3);
+    }
   }
+  __device__ __forceinline__ int kb_group_row(int j) const { return (j * Cfg::NWAVES + wave) * KB_RPG + (int)kb_row; }
   __device__ __forceinline__ int group_row(int j) const { return (j * Cfg::NWAVES + wave) * 8; }
   __device__ __forceinline__ int load_row(int j) const { return group_row(j) + (int)r_in; }
 };
@@ -221,13 +290,15 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
                                                        const uint32_t (&offA)[TileLanes<Cfg>::NJA],
                                                        const uint16_t* const (&baseB)[TileLanes<Cfg>::NJB],
                                                        const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
-                                                       uint8_t* lds, f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
+                                                       uint8_t* lds, f32x16_t (&acc)[Cfg::TM][Cfg::TN],
+                                                       const KMajorB& kb = KMajorB()) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
   constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
   constexpr int L = NJA + NJB;
   constexpr int STAGE = Cfg::STAGE_BYTES, A_BYTES = Cfg::A_BYTES;
   constexpr int NM = TM * TN, ND = TM + TN;
+  constexpr int RB = Cfg::BN * 2;  // K-major weight panel: bytes per row
   const int wave = tl.wave;
 
   auto wave_uniform = [](const uint16_t* p) {
@@ -240,8 +311,22 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
   __amdgpu_buffer_rsrc_t rsA[NJA], rsB[NJB];
 #pragma unroll
   for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseA[j]), 0, 0xffffffff, 0x00020000);
+  if constexpr (!Cfg::B_KMAJOR) {
 #pragma unroll
-  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
+    for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
+  }
+  // K-major: one base per weight, uniform over the wave; the slab offset goes into the base.
+  uint64_t kw[2] = {0, 0};
+  if constexpr (Cfg::B_KMAJOR) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      // readfirstlane returns int: take both halves through uint32_t, or the low half sign-extends
+      const uint64_t v = reinterpret_cast<uint64_t>(kb.w[q]);
+      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+      const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+      kw[q] = ((uint64_t)hi << 32) | lo;
+    }
+  }
 
   uint32_t koff[4];
 #pragma unroll
@@ -250,23 +335,49 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
   uint32_t b_base[TN];
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) b_base[tn] = A_BYTES + (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
+  if constexpr (Cfg::B_KMAJOR) {
+    // This lane's 8 bytes of the first transposing read of K step 0: row 8 * lh + (i >> 2) of the slab,
+    // columns 16 * (group & 1) + 4 * (i & 3) ... of the accumulator tile's 32 (i = lane & 15).
+    const uint32_t i = tl.lane & 15, grp16 = tl.lane >> 4;
+    const uint32_t row = 8 * tl.lh + (i >> 2);
+    const uint32_t key = kmajor_swizzle_key<Cfg::BN>(row);  // K steps and halves add multiples of 4 rows: same key
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const uint32_t unit = (uint32_t)b_frag_row<Cfg>(tl.wn, tn) / 32;
+      b_base[tn] = A_BYTES + row * RB + ((unit ^ key) << 6) + 32 * (grp16 & 1) + 8 * (i & 3);
+    }
+  }
 
   zero_acc<Cfg>(acc);
   const int nk = k_len / kBK;
 
   auto issue_a = [&](int stage, int kt) {
     uint8_t* st = lds + stage * STAGE;
-    const int kb = kt * kRowBytes;
+    const int ko = kt * kRowBytes;
 #pragma unroll
     for (int j = 0; j < NJA; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[j], FFNK_LDS_PTR(st + (j * NWAVES + wave) * 1024), 16, offA[j], kb, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[j], FFNK_LDS_PTR(st + (j * NWAVES + wave) * 1024), 16, offA[j], ko, 0, 0);
+  };
+  // K-major: the slab's resource (weight and slab offset folded into the base, all scalar).
+  auto kmajor_rsrc = [&](int kt) {
+    const int ka = kb.kt_first + kt;
+    const bool second = ka >= kb.kt_switch;
+    const uint64_t base = (second ? kw[1] : kw[0]) + (uint64_t)(uint32_t)(second ? ka - kb.kt_switch : ka) * kb.slab_bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, 0xffffffff, 0x00020000);
   };
   auto issue_b = [&](int stage, int kt) {
     uint8_t* st = lds + stage * STAGE;
-    const int kb = kt * kRowBytes;
+    if constexpr (Cfg::B_KMAJOR) {
+      const __amdgpu_buffer_rsrc_t rs = kmajor_rsrc(kt);
 #pragma unroll
-    for (int j = 0; j < NJB; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[j], FFNK_LDS_PTR(st + A_BYTES + (j * NWAVES + wave) * 1024), 16, offB[j], kb, 0, 0);
+      for (int j = 0; j < NJB; ++j)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, FFNK_LDS_PTR(st + A_BYTES + (j * NWAVES + wave) * 1024), 16, offB[j], 0, 0, 0);
+    } else {
+      const int ko = kt * kRowBytes;
+#pragma unroll
+      for (int j = 0; j < NJB; ++j)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[j], FFNK_LDS_PTR(st + A_BYTES + (j * NWAVES + wave) * 1024), 16, offB[j], ko, 0, 0);
+    }
   };
   auto issue = [&](int stage, int kt) {
     issue_a(stage, kt);
@@ -290,6 +401,84 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
   };
 
+  // ---- K-major weights: the same pipeline written out in source order.  The transposing reads are
+  // asm statements, which scheduling hints cannot place, so every K step is a fixed sequence held by
+  // scheduling barriers: wait for the step's fragments, then its MFMAs with the next step's LDS
+  // reads behind the first ones and (last step of a slab) the global->LDS loads behind the rest. ----
+  constexpr int NR = 2 * TN + TM;                        // LDS reads per K step
+  constexpr int RSLOTS = NM >= 2 ? NM / 2 : 1;
+  constexpr int RPS = (NR + RSLOTS - 1) / RSLOTS;        // reads behind each of the first MFMAs
+  constexpr int RUSED = (NR + RPS - 1) / RPS;
+  constexpr int DPS = (L + (NM - RUSED) - 1) / (NM - RUSED);  // loads behind each of the other MFMAs
+  static_assert(NM > RUSED, "no MFMA left to carry the global->LDS loads");
+  bf16x4_t fb_lo[2][TN], fb_hi[2][TN];  // halves of a weight fragment as the two reads deliver them
+  uint32_t kaddr[2][TN][2];             // LDS address of this lane's reads: [stage][tile][half] (K step: immediate)
+  if constexpr (Cfg::B_KMAJOR) {
+    const uint32_t lds_addr = (uint32_t)reinterpret_cast<uintptr_t>(FFNK_LDS_PTR(lds));
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        kaddr[st][j][0] = lds_addr + st * STAGE + b_base[j];
+        kaddr[st][j][1] = kaddr[st][j][0] + 4 * RB;
+      }
+  }
+  // Reads [r0, r1) of K step `step` of the slab in `stage` into fragment buffer `buf`.
+  auto kmajor_reads = [&](int buf, int stage, auto step, int r0, int r1) {
+    constexpr int ks = decltype(step)::value;
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      if (r < r0 || r >= r1) continue;
+      if (r < 2 * TN) {
+        const bf16x4_t v = lds_read_tr16_b64<16 * ks * RB>(kaddr[stage][r / 2][r & 1]);
+        if (r & 1) fb_hi[buf][r / 2] = v;
+        else fb_lo[buf][r / 2] = v;
+      } else {
+        fa[buf][r - 2 * TN] =
+            *reinterpret_cast<const bf16x8_t*>(lds + stage * STAGE + a_base + (r - 2 * TN) * 32 * kRowBytes + koff[ks]);
+      }
+    }
+  };
+  auto kmajor_step = [&](int cur, int stage_next, auto step_next, bool reads, bool dma, int stage_dma, int kt_dma) {
+    __amdgpu_buffer_rsrc_t rsk = rsA[0];
+    if (dma) rsk = kmajor_rsrc(kt_dma);
+    kmajor_wait_frags<TN>(fb_lo[cur], fb_hi[cur]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[cur][j] = __builtin_shufflevector(fb_lo[cur][j], fb_hi[cur][j], 0, 1, 2, 3, 4, 5, 6, 7);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < NM; ++q) {
+      acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][q % TN], fa[cur][q / TN], acc[q / TN][q % TN], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (q < RUSED) {
+        if (reads) kmajor_reads(cur ^ 1, stage_next, step_next, q * RPS, (q + 1) * RPS);
+      } else if (dma) {
+        uint8_t* st = lds + stage_dma * STAGE;
+#pragma unroll
+        for (int l = (q - RUSED) * DPS; l < (q - RUSED + 1) * DPS && l < L; ++l) {
+          if (l < NJA)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l], FFNK_LDS_PTR(st + (l * NWAVES + wave) * 1024), 16, offA[l],
+                                                     kt_dma * kRowBytes, 0, 0);
+          else
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsk, FFNK_LDS_PTR(st + A_BYTES + ((l - NJA) * NWAVES + wave) * 1024), 16,
+                                                     offB[l - NJA], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  constexpr std::integral_constant<int, 0> s0{};
+  constexpr std::integral_constant<int, 1> s1{};
+  constexpr std::integral_constant<int, 2> s2{};
+  constexpr std::integral_constant<int, 3> s3{};
+  auto kmajor_body = [&](int u, int kt, bool full) {
+    kmajor_step(0, u, s1, true, false, 0, 0);
+    kmajor_step(1, u, s2, true, false, 0, 0);
+    kmajor_step(0, u, s3, true, false, 0, 0);
+    dma_wait_barrier<0>();  // every wave has read the last of stage u; the next slab has landed in the other stage
+    kmajor_step(1, u ^ 1, s0, full || kt + 1 < nk, full || kt + 2 < nk, u, kt + 2);
+  };
+
   // Head of the tile: the weight panels of the first two slabs go out first - their addresses do not
   // depend on the routing - so that they fly while the gathered token rows' indices are still loading.
   issue_b(0, 0);
@@ -301,7 +490,8 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
   } else {
     dma_wait_barrier<0>();
   }
-  load_frags(0, 0, 0);
+  if constexpr (Cfg::B_KMAJOR) kmajor_reads(0, 0, s0, 0, NR);
+  else load_frags(0, 0, 0);
 
   auto body = [&](int u, int kt, bool full) {
     load_frags(1, u, 1);
@@ -329,13 +519,24 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
     }
   };
   int k0 = 0;
-  for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches
-    body(0, k0, true);
-    body(1, k0 + 1, true);
-  }
-  for (; k0 < nk; k0 += 2) {
-    body(0, k0, false);
-    if (k0 + 1 < nk) body(1, k0 + 1, false);
+  if constexpr (Cfg::B_KMAJOR) {
+    for (; k0 + 3 < nk; k0 += 2) {
+      kmajor_body(0, k0, true);
+      kmajor_body(1, k0 + 1, true);
+    }
+    for (; k0 < nk; k0 += 2) {
+      kmajor_body(0, k0, false);
+      if (k0 + 1 < nk) kmajor_body(1, k0 + 1, false);
+    }
+  } else {
+    for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches
+      body(0, k0, true);
+      body(1, k0 + 1, true);
+    }
+    for (; k0 < nk; k0 += 2) {
+      body(0, k0, false);
+      if (k0 + 1 < nk) body(1, k0 + 1, false);
+    }
   }
 #endif
 }
@@ -515,16 +716,33 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
       baseA[j] = a0;
       offA[j] = (uint32_t)((src * g.lda + rl.c_log * 8) * 2);
     }
+    KMajorB kb;
+    if constexpr (Cfg::B_KMAJOR) {
+      // Offsets inside a slab: row of the slab times the row stride, plus this lane's column chunk
+      // (chunks past the last column repeat the last one; their outputs are never stored).
 #pragma unroll
-    for (int j = 0; j < NJB; ++j) {
-      const bool up = Cfg::DUAL && rl.group_row(j) >= BN / 2;  // uniform over the wave
-      const int r = rl.load_row(j) - (up ? BN / 2 : 0);
-      const int n_first = min(n0, g.N - 1);
-      const int n = min(n0 + r, g.N - 1);
-      baseB[j] = (up ? g.B1[grp] : g.B0[grp]) + (int64_t)n_first * g.ldb + k0;
-      offB[j] = (uint32_t)(((int64_t)(n - n_first) * g.ldb + rl.c_log * 8) * 2);
+      for (int j = 0; j < NJB; ++j) {
+        const int n = min(n0 + (int)rl.kb_chunk * 8, g.N - 8);
+        baseB[j] = nullptr;
+        offB[j] = (uint32_t)(((int64_t)rl.kb_group_row(j) * g.ldb + n) * 2);
+      }
+      kb.w[0] = g.B0[grp];
+      kb.w[1] = g.k_switch > 0 ? g.B1[grp] : g.B0[grp];
+      kb.kt_first = kt0;
+      if (g.k_switch > 0) kb.kt_switch = g.k_switch / kBK;
+      kb.slab_bytes = (uint32_t)(g.ldb * (kBK * 2));
+    } else {
+#pragma unroll
+      for (int j = 0; j < NJB; ++j) {
+        const bool up = Cfg::DUAL && rl.group_row(j) >= BN / 2;  // uniform over the wave
+        const int r = rl.load_row(j) - (up ? BN / 2 : 0);
+        const int n_first = min(n0, g.N - 1);
+        const int n = min(n0 + r, g.N - 1);
+        baseB[j] = (up ? g.B1[grp] : g.B0[grp]) + (int64_t)n_first * g.ldb + k0;
+        offB[j] = (uint32_t)(((int64_t)(n - n_first) * g.ldb + rl.c_log * 8) * 2);
+      }
     }
-    if (k_len > 0) gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc);
+    if (k_len > 0) gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
     else zero_acc<Cfg>(acc);  // a range past the end of K contributes exact zeros
     if (!Cfg::DUAL && splits > 1) {
       if (g.tail_mode == 3)  // one compact fp32 tile per (tile, range) pair
@@ -683,6 +901,10 @@ template <class Cfg>
 inline hipError_t launch_routed_gemm(const GemmArgs& g, hipStream_t stream) {
   if (g.M <= 0 || g.N <= 0) return hipSuccess;
   if (g.splits > 1 && (Cfg::DUAL || !Cfg::DIRECT || g.tail_mode != 0 || g.P == nullptr)) return hipErrorInvalidValue;
+  if (Cfg::B_KMAJOR && (g.N % 8 != 0 || g.K % kBK != 0 || g.k_switch % kBK != 0 || g.k_switch < 0 || g.k_switch >= g.K ||
+                        g.ldb * (kBK * 2) + 2 * (int64_t)g.N >= ((int64_t)1 << 32)))
+    return hipErrorInvalidValue;
+  if (!Cfg::B_KMAJOR && g.k_switch != 0) return hipErrorInvalidValue;
   const int grid = routed_gemm_grid<Cfg>(g.M, g.N) * (g.splits > 1 ? g.splits : 1);
   hipLaunchKernelGGL(routed_gemm_kernel<Cfg>, dim3(grid), dim3(Cfg::NT), 0, stream, g);
   return hipGetLastError();

@@ -16,6 +16,15 @@ struct PlainTiles {
   using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupM>;
 };
 
+// The same tiles over K-major weights ([K, N] rows, N contiguous; direct path only).
+template <bool GATHER, bool SCATTER>
+struct KMajorTiles {
+  using T0 = RoutedGemmCfg<256, 256, 2, 4, false, GATHER, SCATTER, true, kGroupM, true>;
+  using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
+  using T2 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
+  using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
+};
+
 // SwiGLU tiles: BN = gate rows + up rows held in LDS, i.e. BN / 2 output columns.
 template <bool DIRECT>
 struct DualTiles {

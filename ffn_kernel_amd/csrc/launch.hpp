@@ -32,6 +32,11 @@ hipError_t launch_up_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t 
 hipError_t launch_down_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream);
 // C(routed order) = route-gather(A) @ B_g^T (MaskedFFN backward: pre-activations, dH)
 hipError_t launch_gather_gemm(int tile, bool direct, const GemmArgs& g, hipStream_t stream);
+// The three single-weight GEMMs above over K-major weights: B0[g] (and B1[g] past GemmArgs::k_switch)
+// is [K, N] rows with N contiguous.  K % 64 == 0 and N % 8 == 0 are required.
+hipError_t launch_linear_gemm_kmajor(int tile, const GemmArgs& g, hipStream_t stream);
+hipError_t launch_down_gemm_kmajor(int tile, const GemmArgs& g, hipStream_t stream);
+hipError_t launch_gather_gemm_kmajor(int tile, const GemmArgs& g, hipStream_t stream);
 // P[grp][split] = A[:, kslice] @ B[:, kslice]^T (fp32 partials; weight gradients)
 hipError_t launch_splitk_gemm(int tile, const SplitKArgs& g, hipStream_t stream);
 

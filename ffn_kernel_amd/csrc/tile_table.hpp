@@ -7,6 +7,7 @@
 #pragma once
 #include "launch.hpp"
 #include "common.hpp"
+#include "gemm_sched.hpp"
 
 namespace ffnk {
 
@@ -43,6 +44,7 @@ inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual) {
 //   time = rounds * (5 us + slabs_per_range * t_slab) + splits * M * n_out * 8 bytes / 4 TB/s
 //   rounds = ceil(tiles * splits / slots),  slots = 256 CUs * workgroups per CU by LDS use,
 //   t_slab = 1.2 us for the 256x256 tile, 0.8 us for the 128x128 and 128x64 tiles.
+// The unsplit 256x256 tile is priced with its split tail (see routed_plan_cost).
 // Limited to M <= 4096 (above it the tiles fill the chip, and the reduce pass launches one row per
 // blockIdx.y); larger M keeps pick_routed_tile and no split.
 struct RoutedPlan {
@@ -57,6 +59,14 @@ inline double routed_plan_cost(int64_t M, int64_t n_out, int64_t K, int tile, in
   const double t_slab = (tile == TILE_256x256_W8 || tile == TILE_256x256_W4) ? 1.2 : 0.8;
   const int64_t slabs = cdiv64(cdiv64(K, 64), splits);
   const double reduce = splits > 1 ? (double)splits * (double)M * (double)n_out * 8.0 / 4.0e6 : 0.0;
+  if (tile == TILE_256x256_W8 && splits == 1 && K % 64 == 0 && tiles > slots) {
+    // Unsplit 256x256 tiles past one round: the launcher runs the whole rounds, then the remaining tiles
+    // cut into K ranges (split tail) - a fraction of a round, a second launch and a small reduce pass.
+    const int64_t tail = tiles % slots;
+    double c = (double)(tiles / slots) * (5.0 + (double)slabs * t_slab);
+    if (tail > 0) c += 15.0 + (double)cdiv64(slabs, tail_split_factor((int)tail, (int)slabs)) * t_slab;
+    return c;
+  }
   return (double)cdiv64(tiles * splits, slots) * (5.0 + (double)slabs * t_slab) + reduce;
 }
 

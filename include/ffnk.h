@@ -198,7 +198,9 @@ FFNK_API int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m,
  * dW1/dW3/dU1/dU3: logical [d, h] with strides (dup_stride_k, dup_stride_n); dW2/dU2: logical
  * [h, d] with strides (ddown_stride_k, ddown_stride_n).  t1, t3, dh, dt1, dt3 and the
  * intermediate are held in bf16 between the GEMMs (the forward does the same for the
- * intermediate); accumulation is fp32; deterministic, no atomics.
+ * intermediate); accumulation is fp32; deterministic, no atomics.  With d and h multiples of 64 and
+ * the weight views the reference passes (or a down weight whose d axis is contiguous) every GEMM reads
+ * the weights in place; other extents and strides are first copied into the workspace.
  * Workspace: ffnk_workspace_bytes(FFNK_OP_FFN_BWD, M, d, h).  Layouts outside the above
  * (d or h not a multiple of 8, unaligned rows, up_stride_k != 1) return FFNK_E_STRIDE.
  */

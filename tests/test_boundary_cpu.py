@@ -68,13 +68,18 @@ def test_tile_table_entries():
     tail = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 72, 1024)
     assert tail["direct_lds"] == 0 and tail["block_k"] == 64 and tail["lds_stages"] == 2
     # few output tiles over a long contraction: the down projection / the linear layer cut K ...
-    for M in (65, 128, 512, 1024, 4096):
+    for M in (65, 128, 512, 1024):
         dn = _lib.tile_config(_lib.OP_FFN_DOWN, M, 4096, 14336)
         assert dn["path"] == _lib.PATH_MFMA_TILED and dn["split_k"] > 1, (M, dn)
         assert (14336 // 64) // dn["split_k"] >= 8  # at least eight slabs per range
         # ... and the workspace holds perm/counts, the [M, h] intermediate and the fp32 partials
         need = M * 4 + 8 + M * 14336 * 2 + dn["split_k"] * M * 4096 * 4
         assert _lib.workspace_bytes(_lib.OP_FFN_FWD, M, 4096, 14336) >= need
+    # just past one round of 256x256 tiles: unsplit, the last partial round runs as a split tail
+    # whose 256 fp32 tiles the workspace holds
+    one = _lib.tile_config(_lib.OP_FFN_DOWN, 4096, 4096, 14336)
+    assert one["split_k"] == 1 and one["block_m"] == 256 and one["block_n"] == 256
+    assert _lib.workspace_bytes(_lib.OP_FFN_FWD, 4096, 4096, 14336) >= 4096 * 4 + 8 + 4096 * 14336 * 2 + 256 * 256 * 256 * 4
     assert _lib.tile_config(_lib.OP_FFN_DOWN, 32768, 4096, 14336)["split_k"] == 1
     assert _lib.tile_config(_lib.OP_FFN_DOWN, 2048, 72, 264)["split_k"] == 1      # K % 64 != 0: no split
     lin = _lib.tile_config(_lib.OP_LINEAR_FWD, 200, 4096, 1024)

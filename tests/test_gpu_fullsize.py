@@ -53,26 +53,26 @@ def test_cfg4_rows_against_c_oracle(cfg4):
 
 
 def test_cfg4_batch_composition_invariance(dev, cfg4):
-    """A row's result does not depend on which other rows share the call: two sequences alone (another
-    tile schedule) reproduce their rows of the full call - bit for bit wherever the K order is shared,
-    i.e. everywhere except the few tiles of a call's last, partial round, which are summed in K ranges;
-    those and a single sequence (4096 rows, whose whole down projection is split over K) agree to bf16
-    accuracy."""
+    """A row's result does not depend on which other rows share the call: two sequences, or one, alone
+    (another tile schedule) reproduce their rows of the full call - bit for bit wherever the K order is
+    shared, i.e. everywhere except the few tiles of a call's last, partial round, which are summed in K
+    ranges; those, and a quarter sequence (1024 rows, whose whole down projection is split over K),
+    agree to bf16 accuracy."""
     note("cfg4 batch invariance")
     w, d, out = cfg4
-    assert _lib.tile_config(_lib.OP_FFN_DOWN, 8192, w.d, w.h)["split_k"] == 1
-    for seq in (0, 5):
-        sl = slice(seq * 4096, (seq + 2) * 4096)
+    for rows in (8192, 4096):
+        assert _lib.tile_config(_lib.OP_FFN_DOWN, rows, w.d, w.h)["split_k"] == 1
+    for sl in (slice(0, 8192), slice(5 * 4096, 7 * 4096), slice(3 * 4096, 4 * 4096)):
         sub = wl.FFNWorkload("seq", d.x[sl].contiguous(), d.W, d.mask[sl].contiguous())
         part = MaskedFFN.apply(*sub.op_args())
         same_rows = (part == out[sl]).all(dim=1).float().mean().item()
-        assert same_rows >= 0.9, same_rows
-        assert_close_bf16_pair(part, out[sl].float().cpu(), "two sequences vs the full call")
-    assert _lib.tile_config(_lib.OP_FFN_DOWN, 4096, w.d, w.h)["split_k"] > 1
-    sl = slice(3 * 4096, 4 * 4096)
+        assert same_rows >= 0.85, same_rows
+        assert_close_bf16_pair(part, out[sl].float().cpu(), "one or two sequences vs the full call")
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 1024, w.d, w.h)["split_k"] > 1
+    sl = slice(3 * 4096, 3 * 4096 + 1024)
     sub = wl.FFNWorkload("seq", d.x[sl].contiguous(), d.W, d.mask[sl].contiguous())
     part = MaskedFFN.apply(*sub.op_args())
-    assert_close_bf16_pair(part, out[sl].float().cpu(), "one sequence (split-K down projection) vs the full call")
+    assert_close_bf16_pair(part, out[sl].float().cpu(), "1024 rows (split-K down projection) vs the full call")
 
 
 def test_cfg4_uniform_sequences_against_library_matmul(dev, cfg4):

@@ -432,6 +432,35 @@ def test_ffn_bwd_vs_oracle(dev, M, d, h, p):
         assert (Wp[k].grad == 0).all()
 
 
+@pytest.mark.parametrize("M,d,h,down_contig", [(300, 256, 512, True), (333, 72, 200, False), (500, 128, 96, False),
+                                               (2100, 512, 1024, True)])
+def test_ffn_bwd_weight_layouts(dev, M, d, h, down_contig):
+    """The backward GEMMs read the weights in place when the layout allows it (the transposed views of
+    [out, in] weights that the reference passes: K-major kernels; a contiguous [h, d] down weight: the
+    forward's kernels) and copy them otherwise (d or h not a multiple of 64).  Same gradients either way."""
+    note(f"ffn bwd layouts M={M} d={d} h={h} down_contig={down_contig}")
+    gen = torch.Generator().manual_seed(M + d + h)
+    mask = torch.rand(M, generator=gen) < 0.5
+    w = wl.make_ffn("t", M, d, h, mask, seed=M + 5, w_std=0.05)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16)
+    dw = w.to(dev)
+    x = dw.x.clone().requires_grad_(True)
+    Wp = {k: v.clone().requires_grad_(True) for k, v in dw.W.items()}
+    # down weights as contiguous [h, d] tensors (stride_n == 1) instead of views of [d, h] ones
+    W2T = {k: Wp[k].T.contiguous().detach().requires_grad_(True) for k in ("w2", "u2")} if down_contig else None
+    dn = (lambda k: W2T[k]) if down_contig else (lambda k: Wp[k].T)
+    out = MaskedFFN.apply(x, Wp["w1"].T, dn("w2"), Wp["w3"].T, Wp["u1"].T, dn("u2"), Wp["u3"].T, dw.mask)
+    out.backward(g.to(dev))
+    torch.cuda.synchronize()
+    dx, dW = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64, round_intermediates=True)
+    assert_close_pipeline(x.grad, dx, "dx")
+    for k in ("w1", "w3", "u1", "u3"):
+        assert_close_pipeline(Wp[k].grad, dW[k], f"d{k}")
+    for k in ("w2", "u2"):
+        got = W2T[k].grad.T if down_contig else Wp[k].grad
+        assert_close_pipeline(got, dW[k], f"d{k}")
+
+
 @pytest.mark.parametrize("M,d,h,p", [(300, 256, 512, 0.5), (1000, 512, 384, 0.3), (777, 128, 320, 1.0), (4500, 1024, 1024, 0.6)])
 def test_ffn_saved_pre_activations(dev, M, d, h, p):
     """A forward that keeps the pre-activations returns the same output, pre-activations that match the
