@@ -89,7 +89,11 @@ BwdPlan plan_bwd(int64_t M, int64_t K, int64_t N, bool dw_k_contig) {
   return p;
 }
 
-// MaskedFFN backward workspace: route | T13 [M, 2h] | DH [M, h] | W2^T, U2^T [h, d] | [W1^T|W3^T],
+// T13 and DH end in 64 rows of padding: the weight-gradient GEMMs load them in whole 64-row slabs (and
+// clear what lies past a group's end before using it).
+constexpr int kBwdPadRows = 64;
+
+// MaskedFFN backward workspace: route | T13 [M + 64, 2h] | DH [M + 64, h] | W2^T, U2^T [h, d] | [W1^T|W3^T],
 // [U1^T|U3^T] [d, 2h] | g^T, x^T [d, ldt] | H^T, dt1^T, dt3^T [h, ldt] | fp32 split-K partials.
 struct FfnBwdPlan {
   BwdPlan up, dn;  // weight-gradient GEMM shapes: up = dW1/dW3 (K = d, N = h), dn = dW2 (K = h, N = d)
@@ -103,8 +107,8 @@ FfnBwdPlan plan_ffn_bwd(int64_t M, int64_t d, int64_t h, bool dup_k_contig, bool
   p.ldt = padded_rows(M);
   const int splits = p.up.tc.splits > p.dn.tc.splits ? p.up.tc.splits : p.dn.tc.splits;
   size_t o = route_ws_bytes(M);
-  p.off_t13 = o;  o += ws_align((size_t)M * 2 * h * 2);
-  p.off_dh = o;   o += ws_align((size_t)M * h * 2);
+  p.off_t13 = o;  o += ws_align((size_t)(M + kBwdPadRows) * 2 * h * 2);
+  p.off_dh = o;   o += ws_align((size_t)(M + kBwdPadRows) * h * 2);
   p.off_w2t = o;  o += 2 * ws_align((size_t)h * d * 2);
   p.off_w13t = o; o += 2 * ws_align((size_t)d * 2 * h * 2);
   p.off_gt = o;   o += ws_align((size_t)d * p.ldt * 2);
@@ -795,13 +799,40 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   if (dxp.splits > 1)
     FFNK_HIP(launch_routed_reduce(b.P, dxp.splits, (int)M, (int)d, r.perm, dx, dx_stride_m, stream), "dx reduce");
 
-  // ---- weight gradients: contraction over the rows of each group, on 64-padded transposes ----
+  // ---- weight gradients: contraction over the rows of each group.  x and g are gathered into
+  // 64-padded transposes; H, dt1 and dt3 (routed order already) are read in place by the K-major
+  // kernels, or transposed as well when their row strides do not fit 32-bit slab offsets. ----
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);    // [d, ldt]
   uint16_t* XT = reinterpret_cast<uint16_t*>(wsb + p.off_xt);    // [d, ldt]
+  float* P = reinterpret_cast<float*>(wsb + p.off_p);
+  const bool in_place = ld13 * 128 + 2 * h < ((int64_t)1 << 32);
+  if (in_place) {
+    FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, x, x_stride_m, (int)d, XT, p.ldt, r.perm, r.counts, (int)M,
+                                      stream, false, false), "g / x transpose");
+    const TileChoice tc = pick_splitk_tile(M, h, d);
+    const int tile = (g_force_tile >= 0 && g_force_tile < TILE_COUNT) ? g_force_tile : tc.tile;
+    // out[r * sr + c * sc]: r runs over h (the in-place operand's columns), c over d
+    auto weight_grad_in_place = [&](const uint16_t* rows, int64_t ld_rows, const uint16_t* cT, uint16_t* o0, uint16_t* o1,
+                                    int64_t sr, int64_t sc) -> int {
+      SplitKArgs s;
+      s.A = rows; s.lda = ld_rows;
+      s.B = cT; s.ldb = p.ldt;
+      s.P = P; s.counts = r.counts; s.M = (int)M;
+      s.R = (int)h; s.Cc = (int)d; s.splits = tc.splits;
+      if (tc.splits == 1) { s.out[0] = o0; s.out[1] = o1; s.out_sr = sr; s.out_sc = sc; }
+      FFNK_HIP(launch_splitk_gemm_kmajor(tile, s, stream), "dW split-K GEMM");
+      if (tc.splits > 1)
+        FFNK_HIP(launch_splitk_reduce(P, tc.splits, (int)h, (int)d, o0, o1, sr, sc, stream), "dW reduce");
+      return FFNK_OK;
+    };
+    if (int e = weight_grad_in_place(DH, h, GT, dW2, dU2, ddown_stride_k, ddown_stride_n)) return e;
+    if (int e = weight_grad_in_place(T13, ld13, XT, dW1, dU1, dup_stride_n, dup_stride_k)) return e;
+    if (int e = weight_grad_in_place(T13 + h, ld13, XT, dW3, dU3, dup_stride_n, dup_stride_k)) return e;
+    return FFNK_OK;
+  }
   uint16_t* HT = reinterpret_cast<uint16_t*>(wsb + p.off_ht);    // [h, ldt]
   uint16_t* D1T = reinterpret_cast<uint16_t*>(wsb + p.off_d1t);  // [h, ldt]
   uint16_t* D3T = reinterpret_cast<uint16_t*>(wsb + p.off_d3t);  // [h, ldt]
-  float* P = reinterpret_cast<float*>(wsb + p.off_p);
   FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, DH, h, (int)h, HT, p.ldt, r.perm, r.counts, (int)M,
                                     stream, false, true), "g / intermediate transpose");
   FFNK_HIP(launch_gather_transpose2(x, x_stride_m, (int)d, XT, T13, ld13, (int)h, D1T, p.ldt, r.perm, r.counts,

@@ -52,6 +52,11 @@ struct GemmArgs {
 // Group grp contracts over columns [k_begin(grp), k_begin(grp) + k_len(grp)) of the two row-major
 // operands; the ranges come from counts[] on the device:
 //   group 0 = [0, pad64(counts[0])),  group 1 = [pad64(counts[0]), + pad64(M - counts[0])).
+// K-major kernels: A is instead the untransposed operand, [M + 64, R] rows in routed order (row stride
+// lda, 16-byte aligned rows, R % 8 == 0); group grp contracts over its rows [counts[0] * grp, ...) in
+// slabs of 64.  The rows of a group's last slab that lie past the group's end (the next group's rows, or
+// the 64 rows of padding the buffer must hold past row M) are loaded and then cleared in LDS: their
+// contents never count.
 struct SplitKArgs {
   const uint16_t* A; int64_t lda;  // [R, Kpad]
   const uint16_t* B; int64_t ldb;  // [Cc, Kpad]

@@ -79,6 +79,9 @@ struct KMajorB {
   int kt_first = 0;                           // first slab of this workgroup's K range
   int kt_switch = 0x7fffffff;
   uint32_t slab_bytes = 0;                    // 64 rows: 64 * ldb * 2
+  // Rows of the range's last slab that belong to the contraction (1..64).  The rest of that slab is
+  // cleared in LDS before it is read, so whatever lies behind the operand's last row never counts.
+  int last_rows = 64;
 };
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool DUAL_, bool GATHER_A_, bool SCATTER_C_,
@@ -467,6 +470,14 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
       __builtin_amdgcn_sched_barrier(0);
     }
   };
+  // Clear rows [last_rows, 64) of the weight panel in `stage` (the range's last slab, after it has landed
+  // and before anyone reads it).  Rows are RB contiguous bytes each, whatever the swizzle inside them.
+  auto kmajor_clear_tail = [&](int stage) {
+    uint8_t* first = lds + stage * STAGE + A_BYTES + kb.last_rows * RB;
+    const int bytes = (kBK - kb.last_rows) * RB;
+    for (int o = (int)threadIdx.x * 16; o < bytes; o += Cfg::NT * 16) *reinterpret_cast<uint4*>(first + o) = make_uint4(0, 0, 0, 0);
+    dma_wait_barrier<0>();
+  };
   constexpr std::integral_constant<int, 0> s0{};
   constexpr std::integral_constant<int, 1> s1{};
   constexpr std::integral_constant<int, 2> s2{};
@@ -476,6 +487,7 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
     kmajor_step(1, u, s2, true, false, 0, 0);
     kmajor_step(0, u, s3, true, false, 0, 0);
     dma_wait_barrier<0>();  // every wave has read the last of stage u; the next slab has landed in the other stage
+    if (!full && kt + 2 == nk && kb.last_rows < kBK) kmajor_clear_tail(u ^ 1);  // never in the steady loop
     kmajor_step(1, u ^ 1, s0, full || kt + 1 < nk, full || kt + 2 < nk, u, kt + 2);
   };
 
@@ -490,8 +502,12 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
   } else {
     dma_wait_barrier<0>();
   }
-  if constexpr (Cfg::B_KMAJOR) kmajor_reads(0, 0, s0, 0, NR);
-  else load_frags(0, 0, 0);
+  if constexpr (Cfg::B_KMAJOR) {
+    if (nk == 1 && kb.last_rows < kBK) kmajor_clear_tail(0);
+    kmajor_reads(0, 0, s0, 0, NR);
+  } else {
+    load_frags(0, 0, 0);
+  }
 
   auto body = [&](int u, int kt, bool full) {
     load_frags(1, u, 1);
@@ -779,7 +795,8 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
 }
 
 // Grouped split-K GEMM of the weight gradients (operands are padded to 64-element slabs, so
-// the direct path always applies).
+// the direct path always applies).  With Cfg::B_KMAJOR the operand A is not a padded transpose but
+// the original [rows, R] matrix in routed order (see SplitKArgs).
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArgs g) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
@@ -830,13 +847,31 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
       baseA[j] = g.B + (int64_t)c_first * g.ldb + k_begin;
       offA[j] = (uint32_t)(((int64_t)(c - c_first) * g.ldb + rl.c_log * 8) * 2);
     }
+    KMajorB kb;
+    if constexpr (Cfg::B_KMAJOR) {
+      // A is read where it lies: contraction rows are its rows (routed order, unpadded), starting at the
+      // group's first routed row.  Rows past the group's end are cleared in LDS (KMajorB::last_rows).
 #pragma unroll
-    for (int j = 0; j < NJB; ++j) {
-      const int r = min(r0 + rl.load_row(j), g.R - 1);
-      baseB[j] = g.A + (int64_t)r_first * g.lda + k_begin;
-      offB[j] = (uint32_t)(((int64_t)(r - r_first) * g.lda + rl.c_log * 8) * 2);
+      for (int j = 0; j < NJB; ++j) {
+        const int r = min(r0 + (int)rl.kb_chunk * 8, g.R - 8);
+        baseB[j] = nullptr;
+        offB[j] = (uint32_t)(((int64_t)rl.kb_group_row(j) * g.lda + r) * 2);
+      }
+      const int64_t row_begin = (grp == 0 ? 0 : n_vis) + (int64_t)kt0 * kBK;
+      kb.w[0] = kb.w[1] = g.A + row_begin * g.lda;
+      kb.slab_bytes = (uint32_t)(g.lda * (kBK * 2));
+      // the group's last slab is ragged: only the range that holds it has rows to clear
+      const int rows_g = grp == 0 ? n_vis : g.M - n_vis;
+      if (kt1 == nk_g) kb.last_rows = rows_g - (nk_g - 1) * kBK;
+    } else {
+#pragma unroll
+      for (int j = 0; j < NJB; ++j) {
+        const int r = min(r0 + rl.load_row(j), g.R - 1);
+        baseB[j] = g.A + (int64_t)r_first * g.lda + k_begin;
+        offB[j] = (uint32_t)(((int64_t)(r - r_first) * g.lda + rl.c_log * 8) * 2);
+      }
     }
-    gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc);
+    gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
   } else {
     zero_acc<Cfg>(acc);  // a split without slabs (e.g. an empty modality) contributes exact zeros
   }
@@ -913,6 +948,7 @@ inline hipError_t launch_routed_gemm(const GemmArgs& g, hipStream_t stream) {
 template <class Cfg>
 inline hipError_t launch_grouped_splitk(const SplitKArgs& g, hipStream_t stream) {
   if (g.R <= 0 || g.Cc <= 0 || g.splits <= 0) return hipSuccess;
+  if (Cfg::B_KMAJOR && (g.R % 8 != 0 || g.lda * (kBK * 2) + 2 * (int64_t)g.R >= ((int64_t)1 << 32))) return hipErrorInvalidValue;
   const int64_t total = 2LL * cdiv(g.R, Cfg::BN) * cdiv(g.Cc, Cfg::BM) * g.splits;
   const int grid = (int)(cdiv64(total, kXcds) * kXcds);
   hipLaunchKernelGGL(grouped_splitk_kernel<Cfg>, dim3(grid), dim3(Cfg::NT), 0, stream, g);

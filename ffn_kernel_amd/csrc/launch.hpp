@@ -39,6 +39,8 @@ hipError_t launch_down_gemm_kmajor(int tile, const GemmArgs& g, hipStream_t stre
 hipError_t launch_gather_gemm_kmajor(int tile, const GemmArgs& g, hipStream_t stream);
 // P[grp][split] = A[:, kslice] @ B[:, kslice]^T (fp32 partials; weight gradients)
 hipError_t launch_splitk_gemm(int tile, const SplitKArgs& g, hipStream_t stream);
+// The same with A read in place: [rows, R] in routed order instead of a padded transpose (SplitKArgs).
+hipError_t launch_splitk_gemm_kmajor(int tile, const SplitKArgs& g, hipStream_t stream);
 
 // ---- prep.hip: layout passes around the GEMMs ----
 // dst[r, c] (row-major, ld_dst) = src[r * sr + c * sc] for r < rows, c < cols.

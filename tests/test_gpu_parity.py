@@ -461,6 +461,36 @@ def test_ffn_bwd_weight_layouts(dev, M, d, h, down_contig):
         assert_close_pipeline(got, dW[k], f"d{k}")
 
 
+def test_ffn_bwd_non_finite_rows_stay_in_their_modality(dev):
+    """The weight-gradient GEMMs load the rows of dt and of the intermediate in 64-row slabs that run past
+    a modality's last row; what lies there (the other modality's rows) must not count - not even as
+    0 * inf.  A non-finite upstream gradient on text rows leaves the visual weights' gradients, and the
+    visual rows of dx, exactly as they are without it."""
+    note("ffn bwd non-finite rows")
+    M, d, h = 333, 128, 256
+    gen = torch.Generator().manual_seed(11)
+    mask = torch.rand(M, generator=gen) < 0.5
+    w = wl.make_ffn("t", M, d, h, mask, seed=4, w_std=0.05).to(dev)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16).to(dev)
+    g_bad = g.clone()
+    g_bad[~w.mask] = float("inf")
+
+    def grads(gg):
+        x = w.x.clone().requires_grad_(True)
+        Wp = {k: v.clone().requires_grad_(True) for k, v in w.W.items()}
+        out = MaskedFFN.apply(x, Wp["w1"].T, Wp["w2"].T, Wp["w3"].T, Wp["u1"].T, Wp["u2"].T, Wp["u3"].T, w.mask)
+        out.backward(gg)
+        torch.cuda.synchronize()
+        return x.grad, {k: v.grad for k, v in Wp.items()}
+
+    dx0, dW0 = grads(g)
+    dx1, dW1 = grads(g_bad)
+    for k in ("w1", "w2", "w3"):
+        assert torch.isfinite(dW1[k]).all() and torch.equal(dW1[k], dW0[k]), k
+    assert torch.equal(dx1[w.mask], dx0[w.mask])
+    assert not torch.isfinite(dW1["u2"]).all()
+
+
 @pytest.mark.parametrize("M,d,h,p", [(300, 256, 512, 0.5), (1000, 512, 384, 0.3), (777, 128, 320, 1.0), (4500, 1024, 1024, 0.6)])
 def test_ffn_saved_pre_activations(dev, M, d, h, p):
     """A forward that keeps the pre-activations returns the same output, pre-activations that match the
