@@ -461,6 +461,36 @@ def test_ffn_bwd_weight_layouts(dev, M, d, h, down_contig):
         assert_close_pipeline(got, dW[k], f"d{k}")
 
 
+def test_ffn_bwd_weights_that_are_slices_of_larger_tensors(dev):
+    """Weights whose rows are longer than the extent used (column slices of wider tensors: row stride >
+    d or h, still 16-byte aligned) are read in place with their own row stride, forward and backward."""
+    note("ffn bwd sliced weights")
+    M, d, h = 700, 256, 384
+    gen = torch.Generator().manual_seed(5)
+    mask = torch.rand(M, generator=gen) < 0.45
+    w = wl.make_ffn("t", M, d, h, mask, seed=9, w_std=0.05)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16)
+    dw = w.to(dev)
+    x = dw.x.clone().requires_grad_(True)
+    wide = {}
+    for k, v in dw.W.items():  # [out, in] weights embedded in [out, in + 64] tensors
+        big = torch.zeros(v.shape[0], v.shape[1] + 64, dtype=v.dtype, device=dev)
+        big[:, 8:8 + v.shape[1]] = v
+        wide[k] = big.requires_grad_(True)
+    view = lambda k: wide[k][:, 8:8 + dw.W[k].shape[1]].T
+    out = MaskedFFN.apply(x, view("w1"), view("w2"), view("w3"), view("u1"), view("u2"), view("u3"), dw.mask)
+    out.backward(g.to(dev))
+    torch.cuda.synchronize()
+    ref = cref.ffn_fwd(w.x, w.W, w.mask, round_mid=True)
+    assert_close(out, ref, "out")
+    dx, dW = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64, round_intermediates=True)
+    assert_close_pipeline(x.grad, dx, "dx")
+    for k in dW:
+        got = wide[k].grad[:, 8:8 + dw.W[k].shape[1]]
+        assert_close_pipeline(got, dW[k], f"d{k}")
+        assert (wide[k].grad[:, :8] == 0).all() and (wide[k].grad[:, 8 + dw.W[k].shape[1]:] == 0).all()
+
+
 def test_ffn_bwd_non_finite_rows_stay_in_their_modality(dev):
     """The weight-gradient GEMMs load the rows of dt and of the intermediate in 64-row slabs that run past
     a modality's last row; what lies there (the other modality's rows) must not count - not even as
