@@ -9,6 +9,11 @@
 // deep (directly, bypassing registers, when K is a multiple of 64; staged through registers
 // otherwise); wavefronts read 16-byte MFMA fragments from an XOR-swizzled LDS layout and issue
 // v_mfma_f32_32x32x16_bf16.
+//
+// The backward GEMMs find one operand with the contraction running over its rows ([K, N], N
+// contiguous: a forward weight seen from the output side, or activations whose rows are summed).
+// RoutedGemmCfg::B_KMAJOR reads such a panel in place: same slabs and stages, the fragments built by
+// the transposing LDS read (see KMajorB).
 #pragma once
 #include <type_traits>
 #include "common.hpp"
