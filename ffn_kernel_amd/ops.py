@@ -8,6 +8,7 @@ Same class names, same positional signatures:
 """
 from __future__ import annotations
 
+import contextlib
 import threading
 
 import torch
@@ -62,6 +63,15 @@ def _same_device(dev, **tensors) -> None:
             raise ValueError(f"{name} is on {t.device}, expected {dev}")
 
 
+_NO_SWITCH = contextlib.nullcontext()
+
+
+def _on_device(dev: torch.device):
+    """Context that makes `dev` the current device; nothing to enter when it already is (the usual case,
+    and the device guard costs several microseconds of a 30 us call)."""
+    return _NO_SWITCH if dev.index is None or torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
+
+
 def _stream_ptr(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
@@ -103,7 +113,7 @@ def masked_linear_forward(a: torch.Tensor, b1: torch.Tensor, b2: torch.Tensor, m
     if M == 0 or N == 0:
         return c
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws_bytes = _lib.workspace_bytes(_lib.OP_LINEAR_FWD, M, K, N)
         ws = _workspace(ws_bytes, dev)
         rc = lib.ffnk_masked_linear_fwd(a.data_ptr(), a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(),
@@ -139,7 +149,7 @@ def masked_linear_backward(grad: torch.Tensor, a: torch.Tensor, b1: torch.Tensor
     if K == 0:
         return da, db1, db2
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws_bytes = _lib.workspace_bytes(_lib.OP_LINEAR_BWD, M, K, N)
         ws = _workspace(ws_bytes, dev)
         rc = lib.ffnk_masked_linear_bwd(grad.data_ptr(), grad.stride(0) if M > 1 else max(N, 1), a.data_ptr(),
@@ -191,7 +201,7 @@ def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre: bool = False):
     pre = None
     if save_pre and h > 0 and lib.ffnk_masked_ffn_can_save(M, d, h) and usk == 1 and dsk == 1:
         pre = torch.empty((M, 2 * h), device=dev, dtype=torch.bfloat16)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_FWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
         head = (a.data_ptr(), a.stride(0) if M > 1 else max(d, 1), ups[0].data_ptr(), ups[1].data_ptr(),
@@ -247,7 +257,7 @@ def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None):
     gusk, gusn = _wstrides(dups[0])
     gdsk, gdsn = _wstrides(ddowns[0])
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
         head = (grad.data_ptr(), grad.stride(0) if M > 1 else d, a.data_ptr(), a.stride(0) if M > 1 else d,
