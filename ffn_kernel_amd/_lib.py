@@ -13,6 +13,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libffnk.so"
 
 OP_LINEAR_FWD, OP_FFN_FWD, OP_LINEAR_BWD, OP_FFN_UP, OP_FFN_DOWN, OP_BWD_DX, OP_BWD_DW, OP_FFN_BWD = range(8)
 PATH_MFMA_TILED, PATH_STREAM, PATH_GENERIC = range(3)
+STATIC_SCRATCH_BYTES = 32 << 20  # FFNK_STATIC_SCRATCH_BYTES
 
 # Every symbol include/ffnk.h declares, with its ctypes signature.
 _SIGNATURES = {
@@ -31,6 +32,9 @@ _SIGNATURES = {
     "ffnk_masked_ffn_fwd_ev": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                        c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64,
                                        c_int64, c_int64, c_void_p, c_size_t, c_void_p, c_void_p]),
+    "ffnk_masked_ffn_fwd_static": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                           c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p,
+                                           c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "ffnk_masked_linear_bwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64,
                                        c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                        c_int64, c_int64, c_void_p, c_size_t, c_void_p]),

@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "common.hpp"
 #include "launch.hpp"
 #include "tile_table.hpp"
@@ -139,6 +141,30 @@ bool kmajor_ok(int64_t K, int64_t N, int64_t ldb, const void* w0, const void* w1
 }
 
 int g_force_tile = -1;  // tuner override, see ffnk_debug_force_tile
+
+// Scratch of ffnk_masked_ffn_fwd_static: one copy per GPU, held from the moment the library's code
+// object is loaded there until the process ends.  The name is a host-side stand-in, not a device
+// address: host code only ever uses the per-device address that static_scratch() looks up.
+static __device__ __align__(256) unsigned char scratch[FFNK_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Address of `scratch` on the current device (looked up once per device; two threads that race
+// here both get the same answer).
+int static_scratch(void** out) {
+  int dev = -1;
+  FFNK_HIP(hipGetDevice(&dev), "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(FFNK_E_SHAPE, "device index %d outside [0, %d)", dev, kMaxDevices);
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    FFNK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    if (p == nullptr) return fail(FFNK_E_NULL, "static scratch has no address on device %d", dev);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return FFNK_OK;
+}
 
 int routed_tile(int64_t M, int64_t n_out, bool dual) {
   return (g_force_tile >= 0 && g_force_tile < TILE_COUNT) ? g_force_tile : pick_routed_tile(M, n_out, dual);
@@ -579,6 +605,25 @@ int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m, const uint16_t
                            int64_t h, void* ws, size_t ws_bytes, void* stream_, void* const* events) {
   return ffn_fwd_impl(x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k, down_stride_n, mask,
                       out, out_stride_m, nullptr, 0, M, d, h, ws, ws_bytes, stream_, events);
+}
+
+int ffnk_masked_ffn_fwd_static(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, const uint16_t* W3,
+                               const uint16_t* U1, const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n,
+                               const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
+                               const uint8_t* mask, uint16_t* out, int64_t out_stride_m, int64_t M, int64_t d,
+                               int64_t h, void* stream_) {
+  if (int e = check_extents(M, d, h)) return e;
+  const size_t need = ffnk_workspace_bytes(FFNK_OP_FFN_FWD, M, d, h);
+  if (need > (size_t)FFNK_STATIC_SCRATCH_BYTES)
+    return fail(FFNK_E_WORKSPACE, "ffnk_masked_ffn_fwd_static: M=%lld d=%lld h=%lld needs %zu bytes of scratch, the static "
+                                  "buffer holds %zu; use ffnk_masked_ffn_fwd with a workspace",
+                (long long)M, (long long)d, (long long)h, need, (size_t)FFNK_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int e = static_scratch(&ws)) return e;
+  // Nothing in the scratch has to start at zero: every region the forward reads (perm, counts, the
+  // intermediate, the fp32 partials) is written by an earlier kernel of the same call.
+  return ffn_fwd_impl(x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k, down_stride_n, mask,
+                      out, out_stride_m, nullptr, 0, M, d, h, ws, (size_t)FFNK_STATIC_SCRATCH_BYTES, stream_, nullptr);
 }
 
 int ffnk_masked_ffn_can_save(int64_t M, int64_t d, int64_t h) {

@@ -164,6 +164,29 @@ FFNK_API int ffnk_masked_ffn_fwd_ev(const uint16_t* x, int64_t x_stride_m,
                            void* ws, size_t ws_bytes, void* stream, void* const* events);
 
 /*
+ * ffnk_masked_ffn_fwd without a workspace argument and without any allocation: for callers that
+ * cannot allocate device memory around the call (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Scratch is a static
+ * device array of FFNK_STATIC_SCRATCH_BYTES inside the library (each GPU the library runs on holds
+ * its own copy until the process ends); shapes whose ffnk_workspace_bytes(FFNK_OP_FFN_FWD, M, d, h)
+ * exceeds that return FFNK_E_WORKSPACE (at d = 4096, h = 14336 every M up to 256 fits).  Same
+ * kernels and results as ffnk_masked_ffn_fwd.  All calls on one GPU share that GPU's array:
+ * calls that overlap on one GPU (different streams or threads) race; calls on one stream are
+ * ordered and safe.  The first call on each GPU looks the array's address up (no allocation); make
+ * that call outside stream capture.
+ */
+#define FFNK_STATIC_SCRATCH_BYTES (32u << 20)
+FFNK_API int ffnk_masked_ffn_fwd_static(const uint16_t* x, int64_t x_stride_m,
+                               const uint16_t* W1, const uint16_t* W3,
+                               const uint16_t* U1, const uint16_t* U3,
+                               int64_t up_stride_k, int64_t up_stride_n,
+                               const uint16_t* W2, const uint16_t* U2,
+                               int64_t down_stride_k, int64_t down_stride_n,
+                               const uint8_t* mask,
+                               uint16_t* out, int64_t out_stride_m,
+                               int64_t M, int64_t d, int64_t h, void* stream);
+
+/*
  * MaskedLinear backward — replaces _bf16_linear_backward (ffn_kernel/linear.py:455-496):
  *   dx[m, :]  = g[m, :] @ (mask[m] ? Wv : Wt)^T
  *   dWv       = x[visual rows]^T @ g[visual rows]       (exact zeros if there are none)
