@@ -42,8 +42,7 @@ def _hipcc() -> str:
 
 def _compile(src: Path) -> Path:
     obj = OBJ_DIR / (src.stem + ".o")
-    extra = os.environ.get("FFNK_HIPCC_FLAGS", "").split()  # developer knob, e.g. -DFFNK_S_UP1=2,4,4,2
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", str(src), "-o", str(obj)]
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)

@@ -38,7 +38,10 @@ int hip_fail(hipError_t e, const char* what) {
     if (e__ != hipSuccess) return hip_fail(e__, what); \
   } while (0)
 
-constexpr int64_t kMaxRows = (int64_t)1 << 30;
+// Row limit: the row partition runs in one launch whose blocks each re-count the mask bytes ahead of
+// their 4096-row chunk (M * M / 8192 bytes of L2 reads in total).  At 2^22 rows that is 2 GB, about
+// half a millisecond; beyond it the quadratic term would dominate the GEMMs it serves.
+constexpr int64_t kMaxRows = (int64_t)1 << 22;
 constexpr int64_t kMaxCols = (int64_t)1 << 24;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -140,7 +143,12 @@ bool kmajor_ok(int64_t K, int64_t N, int64_t ldb, const void* w0, const void* w1
          ldb * 128 + 2 * N < k4g;
 }
 
-int g_force_tile = -1;  // tuner override, see ffnk_debug_force_tile
+std::atomic<int> g_force_tile{-1};  // tuner override, see ffnk_debug_force_tile
+
+int forced_tile() {
+  const int t = g_force_tile.load(std::memory_order_relaxed);
+  return (t >= 0 && t < TILE_COUNT) ? t : -1;
+}
 
 // Scratch of ffnk_masked_ffn_fwd_static: one copy per GPU, held from the moment the library's code
 // object is loaded there until the process ends.  The name is a host-side stand-in, not a device
@@ -167,7 +175,8 @@ int static_scratch(void** out) {
 }
 
 int routed_tile(int64_t M, int64_t n_out, bool dual) {
-  return (g_force_tile >= 0 && g_force_tile < TILE_COUNT) ? g_force_tile : pick_routed_tile(M, n_out, dual);
+  const int f = forced_tile();
+  return f >= 0 ? f : pick_routed_tile(M, n_out, dual);
 }
 
 bool use_stream_path(int64_t M, int64_t d, int64_t h) { return stream_shape_ok(M, d, h); }
@@ -193,8 +202,8 @@ int down_splits(int64_t M, int64_t d, int64_t h) {
 // best split).
 RoutedPlan down_plan(int64_t M, int64_t d, int64_t h) {
   RoutedPlan p;
-  if (g_force_tile >= 0 && g_force_tile < TILE_COUNT) {
-    p.tile = g_force_tile;
+  if (const int f = forced_tile(); f >= 0) {
+    p.tile = f;
     p.splits = pick_routed_splits(M, d, h, p.tile);
   } else {
     p = pick_routed_plan(M, d, h);
@@ -248,9 +257,7 @@ extern "C" {
 int ffnk_version(void) { return FFNK_VERSION; }
 
 int ffnk_debug_force_tile(int tile) {
-  const int prev = g_force_tile;
-  g_force_tile = (tile >= 0 && tile < TILE_COUNT) ? tile : -1;
-  return prev;
+  return g_force_tile.exchange((tile >= 0 && tile < TILE_COUNT) ? tile : -1);
 }
 
 const char* ffnk_last_error(void) { return g_err; }
@@ -855,7 +862,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
     FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, x, x_stride_m, (int)d, XT, p.ldt, r.perm, r.counts, (int)M,
                                       stream, false, false), "g / x transpose");
     const TileChoice tc = pick_splitk_tile(M, h, d);
-    const int tile = (g_force_tile >= 0 && g_force_tile < TILE_COUNT) ? g_force_tile : tc.tile;
+    const int tile = forced_tile() >= 0 ? forced_tile() : tc.tile;
     // out[r * sr + c * sc]: r runs over h (the in-place operand's columns), c over d
     auto weight_grad_in_place = [&](const uint16_t* rows, int64_t ld_rows, const uint16_t* cT, uint16_t* o0, uint16_t* o1,
                                     int64_t sr, int64_t sc) -> int {

@@ -243,12 +243,6 @@ __global__ __launch_bounds__(256) void stream_reduce_kernel(const float* __restr
 // Shape of the streaming kernel per (m-tiles, projection): RT row tiles of 16 weight rows per
 // wavefront (a token-row fragment is then used RT times), KS 32-element k-steps per chunk, NWV
 // wavefronts per workgroup sharing the K range, OCC waves per SIMD the register budget allows.
-#ifndef FFNK_S_UP1
-#define FFNK_S_UP1 1, 4, 4, 4
-#endif
-#ifndef FFNK_S_DOWN1
-#define FFNK_S_DOWN1 1, 4, 16, 4
-#endif
 template <int RT_, int KS_, int NWV_, int OCC_>
 struct StreamShapeV {
   static constexpr int RT = RT_, KS = KS_, NWV = NWV_, OCC = OCC_;
@@ -256,9 +250,9 @@ struct StreamShapeV {
 template <int NTM_MAX, bool DUAL>
 struct StreamShape : StreamShapeV<2, (DUAL ? 2 : 4), 4, 2> {};
 template <>
-struct StreamShape<1, true> : StreamShapeV<FFNK_S_UP1> {};
+struct StreamShape<1, true> : StreamShapeV<1, 4, 4, 4> {};
 template <>
-struct StreamShape<1, false> : StreamShapeV<FFNK_S_DOWN1> {};
+struct StreamShape<1, false> : StreamShapeV<1, 4, 16, 4> {};
 
 int stream_rows_per_block(int M, bool dual) {
   switch (cdiv(M, 16)) {

@@ -37,13 +37,10 @@ constexpr int kTK = 128;    // K elements per chunk (16 pieces of 16 bytes per r
 // Shape per number of 16-row m-tiles the call can have (ceil(M / 16)): wavefronts per workgroup
 // (sharing one token-row slab; fewer wavefronts = less barrier coupling and more workgroups, but
 // every thread then stages more of the slab) and chunks in flight per wavefront (register budget).
-#ifndef FFNK_TILE_SHAPES
-#define FFNK_TILE_SHAPES {2, 4, 0}, {2, 3, 0}, {2, 3, 1}, {2, 3, 1}
-#endif
 // dma: the token-row slab is filled by direct global -> LDS loads (no staging registers, which is
 // what lets the 3- and 4-m-tile shapes run two-wavefront workgroups) instead of through registers.
 struct TileShapeEntry { int waves, depth, dma; };
-constexpr TileShapeEntry kTileShapes[4] = {FFNK_TILE_SHAPES};
+constexpr TileShapeEntry kTileShapes[4] = {{2, 4, 0}, {2, 3, 0}, {2, 3, 1}, {2, 3, 1}};
 constexpr int kTMaxM = 64;
 
 struct TileJob {

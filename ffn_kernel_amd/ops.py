@@ -40,10 +40,18 @@ def _require_mask(mask: torch.Tensor, M: int, dev: torch.device) -> torch.Tensor
 
 
 def _rows_contiguous(t: torch.Tensor) -> torch.Tensor:
-    """[M, K] with unit column stride (what the reference's a.contiguous() guarantees,
-    linear.py:430) — row-strided views are passed through without a copy."""
-    if t.shape[1] <= 1 or t.stride(1) == 1:
-        if t.shape[0] <= 1 or t.stride(0) >= t.shape[1]:
+    """[M, K] rows the MFMA kernels can address: unit column stride, and - when K is a multiple of 8,
+    i.e. when the fast path applies at all - a row stride that is a multiple of 8 elements on a
+    16-byte aligned base.  Such views pass through without a copy; anything else is copied, as the
+    reference's a.contiguous() / gd.contiguous() does for every input (linear.py:430, 463;
+    ffn.py:533), so that an odd view never drops onto the slow any-stride kernels."""
+    M, K = t.shape
+    unit_cols = K <= 1 or t.stride(1) == 1
+    rows_ok = M <= 1 or t.stride(0) >= K
+    if unit_cols and rows_ok:
+        if K % 8 != 0 or K == 0:
+            return t  # the any-stride kernels take it as it is; a copy would not change the path
+        if (M <= 1 or t.stride(0) % 8 == 0) and t.data_ptr() % 16 == 0:
             return t
     return t.contiguous()
 

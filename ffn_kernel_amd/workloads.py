@@ -179,3 +179,18 @@ def cfg5_ffn_decode(M: int, kind: str = "bernoulli", seed: int = 0, d: int = 409
     else:
         raise ValueError(kind)
     return make_ffn(f"cfg5_ffn_decode_M{M}_{kind}_d{d}_h{h}", M, d, h, mask, seed)
+
+
+def cfg5_inputs(M: int, kind: str = "bernoulli", seed: int = 0, d: int = 4096):
+    """(x, mask) of cfg5_ffn_decode(M, kind, seed) without generating its weights (x is the first draw of
+    that workload's generator), for callers that bring their own weight sets."""
+    w_gen = torch.Generator().manual_seed(seed)
+    x = _randn_bf16((M, d), 1.0, w_gen)
+    gen = torch.Generator().manual_seed(5000 + seed + 17 * M)
+    if kind == "bernoulli":
+        mask = bernoulli_mask(M, 0.5, gen)
+    elif kind in ("visual", "text"):
+        mask = torch.full((M,), kind == "visual", dtype=torch.bool)
+    else:
+        raise ValueError(kind)
+    return x, mask

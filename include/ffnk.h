@@ -101,10 +101,12 @@ FFNK_API size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N);
 FFNK_API int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t* out);
 
 /*
- * Tuning hook: force every LDS-tiled GEMM launched by this process to use tile id `tile`
+ * Tuner-only hook: force every LDS-tiled GEMM launched by this process to use tile id `tile`
  * (0 = 256x256 / 8 waves, 1 = 256x256 / 4 waves, 2 = 128x128 / 4 waves, 3 = small), or -1 to
- * return to the tile table.  Process-global; meant for the tuner (python -m ffn_kernel_amd.tune),
- * which plays the role of the reference's find_spec table lookups.  Returns the previous value.
+ * return to the tile table.  The one piece of process-global state in the library (an atomic int
+ * read at every launch): it exists for the tuner (python -m ffn_kernel_amd.tune, the counterpart of
+ * the reference's find_spec/*.py sweeps) and for tests that run every compiled tile; production
+ * callers leave it alone.  Returns the previous value.
  */
 FFNK_API int ffnk_debug_force_tile(int tile);
 

@@ -177,3 +177,15 @@ def test_workloads_are_seeded_and_shaped():
     nv = int(c5b.mask.sum())
     assert c5b.algorithmic_bytes() == 3 * 64 * 128 * 2 * (int(nv > 0) + int(nv < 8)) + 2 * 8 * 64 * 2 + 8
     assert wl.cfg2_ffn_fwd().routed_flops == 2 * 8192 * 1024 * 2048 * 3
+
+
+def test_reference_import_name_resolves():
+    """The reference's import line (ffn_kernel/__init__.py:1, README.md:46, 81) works unchanged."""
+    from ffn_kernel import MaskedFFN as F2, MaskedLinear as L2
+    assert L2 is MaskedLinear and F2 is MaskedFFN
+
+
+def test_row_limit_is_what_one_route_launch_handles():
+    assert _lib.workspace_bytes(_lib.OP_LINEAR_FWD, 1 << 22, 64, 64) > 0
+    with pytest.raises(ValueError):
+        _lib.workspace_bytes(_lib.OP_LINEAR_FWD, (1 << 22) + 1, 64, 64)

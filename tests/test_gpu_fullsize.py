@@ -95,6 +95,30 @@ def test_cfg4_uniform_sequences_against_library_matmul(dev, cfg4):
     assert checked >= 2
 
 
+def test_cfg4_mixed_sequences_every_row(dev, cfg4):
+    """The sequences that mix visual and text tokens (visual fraction 0.3 / 0.7) are the routed case:
+    every one of their rows is checked against the select form in fp32 library matmuls on the GPU."""
+    note("cfg4 mixed sequences, every row")
+    w, d, out = cfg4
+    per_seq = w.mask.reshape(8, 4096).sum(1)
+    checked = 0
+    for seq in range(8):
+        if per_seq[seq] in (0, 4096):
+            continue
+        sl = slice(seq * 4096, (seq + 1) * 4096)
+        x = d.x[sl].float()
+        m = d.mask[sl]
+        ref = torch.empty(4096, w.d, device=dev, dtype=torch.float32)
+        for sel, (k1, k2, k3) in ((m, ("w1", "w2", "w3")), (~m, ("u1", "u2", "u3"))):
+            t1 = x[sel] @ d.W[k1].float().T
+            t3 = x[sel] @ d.W[k3].float().T
+            hmid = (t1 * torch.sigmoid(t1) * t3).to(torch.bfloat16).float()
+            ref[sel] = hmid @ d.W[k2].float().T
+        assert_close(out[sl], ref.double().cpu(), f"mixed sequence {seq} ({int(per_seq[seq])} visual rows)")
+        checked += 1
+    assert checked >= 2
+
+
 def test_ffn_split_tail_of_the_down_projection(dev):
     """8500 rows x 4096 output columns: 34 or 35 row tiles x 16 column tiles of 256x256, i.e. two whole
     rounds of 256 tiles and a remainder that runs cut into K ranges with a reduce pass.  Checked against
@@ -144,7 +168,8 @@ def test_linear_fullsize_scaling_is_exact(dev):
     assert torch.equal(y2, y1 * 2)
 
 
-@pytest.mark.parametrize("M,kind", [(1, "visual"), (1, "text"), (8, "bernoulli"), (64, "bernoulli")])
+@pytest.mark.parametrize("M,kind", [(1, "visual"), (1, "text"), (8, "bernoulli"), (32, "bernoulli"), (64, "bernoulli"),
+                                    (32, "visual"), (64, "text")])
 def test_cfg5_decode_fullsize(dev, M, kind):
     """Decode path at d=4096, h=14336: agrees with the tiled path on the same rows (embedded in a
     65-row call, which the tile table sends to the GEMM kernels), and never reads an absent modality."""

@@ -11,6 +11,7 @@ import torch
 
 from ffn_kernel_amd import MaskedFFN, MaskedLinear, _lib
 from ffn_kernel_amd import workloads as wl
+from ffn_kernel_amd.ops import masked_ffn_backward, masked_ffn_forward, masked_linear_backward
 from oracle import cref
 from oracle import modules as om
 from helpers import assert_close, assert_close_bf16_pair, assert_close_pipeline, note
@@ -751,3 +752,102 @@ def test_ffn_forward_keeps_pre_activations_only_when_a_backward_can_follow(dev, 
     out = MaskedFFN.apply(x, *args[1:])                      # training
     out.sum().backward()
     assert seen == [False, False, True] and x.grad is not None
+
+
+# ------------------------------------------------------------------ every compiled tile, forced
+@pytest.fixture
+def force_tile():
+    """ffnk_debug_force_tile for the duration of one test; always back to the tile table afterwards."""
+    lib = _lib.load()
+    try:
+        yield lib.ffnk_debug_force_tile
+    finally:
+        lib.ffnk_debug_force_tile(-1)
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("M,K,N,p", [(700, 256, 512, 0.5), (333, 192, 320, 0.3), (1100, 1024, 264, 1.0)])
+def test_forced_tile_linear_fwd_bwd(dev, force_tile, tile, M, K, N, p):
+    """Each of the four tile shapes every GEMM family is compiled for (256x256 with 8 or 4 waves,
+    128x128, 128x64) runs the MaskedLinear forward and backward: the table alone never picks all of
+    them at test sizes."""
+    note(f"forced tile {tile}: linear fwd+bwd M={M} K={K} N={N} p={p}")
+    gen = torch.Generator().manual_seed(M + tile)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_linear("t", M, K, N, mask, seed=M + K, with_grad=True, w_std=0.05)
+    dw = w.to(dev)
+    force_tile(tile)
+    y = MaskedLinear.apply(dw.x, dw.Wv.T, dw.Wt.T, dw.mask)
+    dx, dWv, dWt = masked_linear_backward(dw.grad, dw.x, dw.Wv.T, dw.Wt.T, dw.mask)
+    torch.cuda.synchronize()
+    force_tile(-1)
+    assert_close(y, cref.linear_fwd(w.x, w.Wv, w.Wt, w.mask), "y")
+    rdx, rdWv, rdWt = cref.linear_bwd(w.grad, w.x, w.Wv, w.Wt, w.mask)
+    assert_close(dx, rdx, "dx")
+    assert_close(dWv.T, rdWv, "dWv")
+    assert_close(dWt.T, rdWt, "dWt")
+    if p == 1.0:
+        assert torch.count_nonzero(dWt) == 0
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("M,d,h,p", [(700, 256, 512, 0.5), (300, 128, 320, 0.4)])
+def test_forced_tile_ffn_fwd_bwd(dev, force_tile, tile, M, d, h, p):
+    note(f"forced tile {tile}: ffn fwd+bwd M={M} d={d} h={h}")
+    gen = torch.Generator().manual_seed(M + tile)
+    mask = torch.rand(M, generator=gen) < p
+    w = wl.make_ffn("t", M, d, h, mask, seed=M + 3, w_std=0.05)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16)
+    dw = w.to(dev)
+    force_tile(tile)
+    out, pre = masked_ffn_forward(*dw.op_args(), save_pre=True)
+    grads_saved = masked_ffn_backward(g.to(dev), *dw.op_args(), pre=pre)
+    grads = masked_ffn_backward(g.to(dev), *dw.op_args())
+    torch.cuda.synchronize()
+    force_tile(-1)
+    assert_close(out, cref.ffn_fwd(w.x, w.W, w.mask, round_mid=True), "ffn out")
+    rdx, rdW = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64, round_intermediates=True)
+    for got in (grads, grads_saved):
+        assert_close_pipeline(got[0], rdx, "dx")
+        for i, k in enumerate(("w1", "w2", "w3", "u1", "u2", "u3")):
+            assert_close_pipeline(got[1 + i].T, rdW[k], f"d{k}")
+
+
+def test_ffn_fwd_bwd_on_unaligned_views(dev):
+    """x and the upstream gradient as column slices of wider tensors whose row stride is not a multiple
+    of 8 elements and whose first element is not 16-byte aligned: the ops copy such views (as the
+    reference's .contiguous() calls do) instead of handing them to a kernel that cannot address them."""
+    note("ffn fwd+bwd on unaligned column-sliced x and grad")
+    M, d, h = 300, 256, 512
+    gen = torch.Generator().manual_seed(77)
+    mask = torch.rand(M, generator=gen) < 0.5
+    w = wl.make_ffn("t", M, d, h, mask, seed=78, w_std=0.05)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16)
+    dw = w.to(dev)
+    wide_x = torch.zeros(M, d + 100, dtype=torch.bfloat16, device=dev)
+    wide_x[:, 4:4 + d] = dw.x
+    wide_g = torch.zeros(M, d + 36, dtype=torch.bfloat16, device=dev)
+    wide_g[:, 3:3 + d] = g.to(dev)
+    x = wide_x[:, 4:4 + d].detach().requires_grad_(True)
+    Wp = {k: v.clone().requires_grad_(True) for k, v in dw.W.items()}
+    out = MaskedFFN.apply(x, Wp["w1"].T, Wp["w2"].T, Wp["w3"].T, Wp["u1"].T, Wp["u2"].T, Wp["u3"].T, dw.mask)
+    out.backward(wide_g[:, 3:3 + d])
+    torch.cuda.synchronize()
+    assert_close(out, cref.ffn_fwd(w.x, w.W, w.mask, round_mid=True), "out")
+    rdx, rdW = om.ffn_backward_select(g, w.x, w.W, w.mask, torch.float64, round_intermediates=True)
+    assert_close_pipeline(x.grad, rdx, "dx")
+    for k in rdW:
+        assert_close_pipeline(Wp[k].grad, rdW[k], f"d{k}")
+    # the same views through MaskedLinear: forward and backward stay on the MFMA path's results
+    lw = wl.make_linear("t", M, d, 192, mask, seed=79, with_grad=True, w_std=0.05)
+    dl = lw.to(dev)
+    wide_x[:, 4:4 + d] = dl.x
+    wide_gl = torch.zeros(M, 192 + 4, dtype=torch.bfloat16, device=dev)
+    wide_gl[:, 1:193] = dl.grad
+    y = MaskedLinear.apply(wide_x[:, 4:4 + d], dl.Wv.T, dl.Wt.T, dl.mask)
+    dx, dWv, dWt = masked_linear_backward(wide_gl[:, 1:193], wide_x[:, 4:4 + d], dl.Wv.T, dl.Wt.T, dl.mask)
+    assert_close(y, cref.linear_fwd(lw.x, lw.Wv, lw.Wt, lw.mask), "linear y")
+    rdx, rdWv, rdWt = cref.linear_bwd(lw.grad, lw.x, lw.Wv, lw.Wt, lw.mask)
+    assert_close(dx, rdx, "linear dx")
+    assert_close(dWv.T, rdWv, "linear dWv")
+    assert_close(dWt.T, rdWt, "linear dWt")
