@@ -234,7 +234,7 @@ RoutedPlan linear_plan(int64_t M, int64_t K, int64_t N) {
 size_t linear_partial_bytes(int64_t M, int64_t K, int64_t N) {
   const RoutedPlan p = linear_plan(M, K, N);
   if (p.splits > 1) return ws_align((size_t)p.splits * M * N * 4);
-  if (p.tile == TILE_256x256_W8 && K % 64 == 0) return ws_align((size_t)kTailSlots * 256 * 256 * 4);
+  if (is_big_tile(p.tile) && K % 64 == 0) return ws_align((size_t)kTailSlots * 256 * 256 * 4);
   return 0;
 }
 int down_tile(int64_t M, int64_t d, int64_t h) { return down_plan(M, d, h).tile; }
@@ -246,7 +246,7 @@ int tiled_down_splits(int64_t M, int64_t d, int64_t h) {
 size_t tiled_down_partial_bytes(int64_t M, int64_t d, int64_t h) {
   const RoutedPlan p = down_plan(M, d, h);
   if (p.splits > 1) return ws_align((size_t)p.splits * M * d * 4);
-  if (p.tile == TILE_256x256_W8 && h % 64 == 0) return ws_align((size_t)kTailSlots * 256 * 256 * 4);
+  if (is_big_tile(p.tile) && h % 64 == 0) return ws_align((size_t)kTailSlots * 256 * 256 * 4);
   return 0;
 }
 
@@ -453,7 +453,7 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
   if (plan.splits > 1) {
     g.splits = plan.splits;
     g.P = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + r.bytes);
-  } else if (direct && plan.tile == TILE_256x256_W8) {
+  } else if (direct && is_big_tile(plan.tile)) {
     g.P_tail = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + r.bytes);
   }
   FFNK_HIP(launch_linear_gemm(plan.tile, direct, g, stream), "linear GEMM");
@@ -591,7 +591,7 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
   if (dn_splits > 1) {
     dn.splits = dn_splits;
     dn.P = partials;
-  } else if (dn_direct && down_tile(M, d, h) == TILE_256x256_W8) {
+  } else if (dn_direct && is_big_tile(down_tile(M, d, h))) {
     dn.P_tail = partials;  // the last, partial round of 256x256 tiles runs cut into K ranges
   }
   FFNK_HIP(launch_down_gemm(down_tile(M, d, h), dn_direct, dn, stream), "down-projection GEMM");
@@ -842,7 +842,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   if (dxp.splits > 1) {
     b.splits = dxp.splits;
     b.P = reinterpret_cast<float*>(wsb + p.off_w2t);
-  } else if (dx_direct && dxp.tile == TILE_256x256_W8 &&
+  } else if (dx_direct && is_big_tile(dxp.tile) &&
              (size_t)kTailSlots * 256 * 256 * 4 <= 2 * ws_align((size_t)h * d * 2)) {
     b.P_tail = reinterpret_cast<float*>(wsb + p.off_w2t);  // split tail of the last, partial round
   }

@@ -52,14 +52,9 @@ inline hipError_t dispatch_tile(int tile, const GemmArgs& g, hipStream_t stream)
 // schedule - same K order per output element, so the result does not depend on which launch computed
 // it - or, with GemmArgs::P_tail, on the big tile cut into K ranges plus a reduce pass (another
 // summation order for the rows of those tiles, a shorter tail: 0.20 -> 0.05 ms at the shape above).
-template <class Tiles>
-inline hipError_t dispatch_tile_with_tail(int tile, const GemmArgs& g, hipStream_t stream) {
-  using Big = typename Tiles::T0;
+template <class Tiles, class Big>
+inline hipError_t dispatch_big_tile_with_tail(const GemmArgs& g, hipStream_t stream) {
   using Small = typename Tiles::T2;
-  if (tile != TILE_256x256_W8 || g.splits > 1 || g.M <= 0 || g.N <= 0) return dispatch_tile<Tiles>(tile, g, stream);
-  // At most one round of big tiles: nothing to split off (every tile would land in the remainder).
-  if ((int64_t)(cdiv(g.M, Tiles::T0::BM) + 1) * cdiv(g.N, Tiles::T0::BN_OUT) <= kCusPerChip)
-    return dispatch_tile<Tiles>(tile, g, stream);
   GemmArgs a = g;
   a.tail_mode = 1;
   if (hipError_t e = launch_routed_gemm<Big>(a, stream)) return e;
@@ -78,6 +73,16 @@ inline hipError_t dispatch_tile_with_tail(int tile, const GemmArgs& g, hipStream
   constexpr int q = (Big::BM / Small::BM) * (Big::BN_OUT / Small::BN_OUT);
   hipLaunchKernelGGL(routed_gemm_kernel<Small>, dim3((kCusPerChip - 1) * q), dim3(Small::NT), 0, stream, a);
   return hipGetLastError();
+}
+
+template <class Tiles>
+inline hipError_t dispatch_tile_with_tail(int tile, const GemmArgs& g, hipStream_t stream) {
+  if (!is_big_tile(tile) || g.splits > 1 || g.M <= 0 || g.N <= 0) return dispatch_tile<Tiles>(tile, g, stream);
+  // At most one round of big tiles: nothing to split off (every tile would land in the remainder).
+  if ((int64_t)(cdiv(g.M, Tiles::T0::BM) + 1) * cdiv(g.N, Tiles::T0::BN_OUT) <= kCusPerChip)
+    return dispatch_tile<Tiles>(tile, g, stream);
+  return tile == TILE_256x256_W8 ? dispatch_big_tile_with_tail<Tiles, typename Tiles::T0>(g, stream)
+                                 : dispatch_big_tile_with_tail<Tiles, typename Tiles::T1>(g, stream);
 }
 
 }  // namespace ffnk

@@ -18,6 +18,9 @@ enum TileId : int {
   TILE_COUNT = 4
 };
 
+// The two 256x256 tiles: past one round of the chip they run whole rounds first and the remainder apart.
+inline bool is_big_tile(int tile) { return tile == TILE_256x256_W8 || tile == TILE_256x256_W4; }
+
 // Geometry of a tile id, as reported through ffnk_tile_config().
 struct TileGeom {
   int block_m, block_n_out, waves_m, waves_n;
