@@ -107,12 +107,19 @@ struct RoutedGemmCfg {
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int NT = NWAVES * kWave;
   // One wavefront per SIMD: the K loop is a fixed, source-order schedule (see gemm_mainloop_slab_dma).
-  static constexpr bool FIXED_SCHEDULE = DIRECT_ && !B_KMAJOR_ && BM_ == 256;
+  static constexpr bool FIXED_SCHEDULE = DIRECT_ && !B_KMAJOR_ && BM_ == 256;  // (32x32x16 form; superseded where MFMA16)
   static constexpr int BN_OUT = DUAL ? BN / 2 : BN;        // output columns per tile
   static constexpr int WTM = BM / WAVES_M;                 // rows per wave
   static constexpr int WTN_OUT = BN_OUT / WAVES_N;         // output columns per wave
-  static constexpr int TM = WTM / 32;                      // 32x32 MFMA tiles per wave, M direction
-  static constexpr int TN_OUT = WTN_OUT / 32;
+  // The 256-row direct tiles accumulate with v_mfma_f32_16x16x32_bf16 (four accumulator registers read
+  // and written per 16 K-products of a lane instead of sixteen per 16: the kernel runs at the board's
+  // power limit and the narrower accumulator traffic is worth 5 % there); the others with 32x32x16.
+  static constexpr bool MFMA16 = DIRECT_ && !B_KMAJOR_ && BM_ == 256;
+  static constexpr int MT = MFMA16 ? 16 : 32;              // edge of an accumulator tile
+  static constexpr int ACC_N = MT * MT / kWave;            // accumulator registers per tile
+  using Acc = std::conditional_t<MFMA16, f32x4_t, f32x16_t>;
+  static constexpr int TM = WTM / MT;                      // accumulator tiles per wave, M direction
+  static constexpr int TN_OUT = WTN_OUT / MT;
   static constexpr int TN = DUAL ? 2 * TN_OUT : TN_OUT;    // accumulator tiles per wave, N direction
   static constexpr int A_BYTES = BM * kRowBytes;           // slab layout
   static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
@@ -127,18 +134,27 @@ struct RoutedGemmCfg {
 // Accumulator tile b of the wave reads B-panel rows starting here.
 template <class Cfg>
 __device__ __forceinline__ int b_frag_row(int wn, int tn) {
-  if (Cfg::DUAL) return (tn < Cfg::TN_OUT ? 0 : Cfg::BN / 2) + wn * Cfg::WTN_OUT + (tn % Cfg::TN_OUT) * 32;
-  return wn * Cfg::WTN_OUT + tn * 32;
+  if (Cfg::DUAL) return (tn < Cfg::TN_OUT ? 0 : Cfg::BN / 2) + wn * Cfg::WTN_OUT + (tn % Cfg::TN_OUT) * Cfg::MT;
+  return wn * Cfg::WTN_OUT + tn * Cfg::MT;
 }
 
 template <class Cfg>
-__device__ __forceinline__ void zero_acc(f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
+__device__ __forceinline__ void zero_acc(typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN]) {
 #pragma unroll
   for (int i = 0; i < Cfg::TM; ++i)
 #pragma unroll
     for (int j = 0; j < Cfg::TN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+      for (int v = 0; v < Cfg::ACC_N; ++v) acc[i][j][v] = 0.f;
+}
+
+// Where element v of an accumulator tile lies: the lane holds token row `lr` of the tile (the MFMA's
+// second operand) and, of the tile's weight rows (= output columns), those at acc_col(v, lh):
+//   32x32x16: lr = lane & 31, lh = lane >> 5, columns 8 * (v / 4) + 4 * lh + v % 4
+//   16x16x32: lr = lane & 15, lh = lane >> 4, columns 4 * lh + v
+template <class Cfg>
+__device__ __forceinline__ constexpr int acc_col(int v, int lh) {
+  return Cfg::MT == 32 ? 8 * (v / 4) + 4 * lh + (v % 4) : 4 * lh + v;
 }
 
 constexpr int waitcnt_imm(int vm, int lgkm) {  // gfx9 s_waitcnt encoding, expcnt untouched
@@ -166,7 +182,7 @@ struct TileLanes {
   int wave_s;      // the wave index again, held in a scalar register (LDS destinations of the global->LDS loads)
   uint32_t r_in;   // row inside the 8-row group this lane loads
   uint32_t c_log;  // logical 16-byte chunk (0..7) of that row
-  uint32_t lr, lh; // MFMA fragment row (0..31) and K half (0..1)
+  uint32_t lr, lh; // MFMA fragment row (0 .. MT-1) and 8-element K piece of the lane (0..1 or 0..3)
   // K-major weight panel: a 64-row slab of BN-element rows is moved as 1 KB groups of 64 / (BN / 8)
   // whole rows; this lane fills physical slot `lane` of its group, which holds logical chunk kb_chunk
   // of row kb_row of the group.
@@ -186,8 +202,8 @@ struct TileLanes {
     const uint32_t q = lane & 15;
     r_in = 2 * (lane >> 4) + ((q >> 3) ^ (wave & 1));
     c_log = (q & 7) ^ r_in;
-    lr = lane & 31;
-    lh = lane >> 5;
+    lr = lane & (Cfg::MT - 1);
+    lh = lane / Cfg::MT;
     kb_row = kb_chunk = 0;
     if (Cfg::B_KMAJOR) {
       static_assert(!Cfg::B_KMAJOR || (KB_CPR <= 64 && (KB_RPG == 2 || KB_RPG == 4 || KB_RPG == 8)), "BN of 64, 128 or 256");
@@ -212,7 +228,8 @@ template <class Cfg>
 __device__ __forceinline__ void gemm_mainloop_staged(const TileLanes<Cfg>& tl,
                                                      const uint16_t* const (&pa)[TileLanes<Cfg>::NJA],
                                                      const uint16_t* const (&pb)[TileLanes<Cfg>::NJB], int k_len,
-                                                     uint8_t* lds, f32x16_t (&acc)[Cfg::TM][Cfg::TN]) {
+                                                     uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN]) {
+  static_assert(!Cfg::MFMA16, "the register-staged loop issues 32x32x16 MFMAs");
   constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
   constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
   const int lane = tl.lane, wave = tl.wave;
@@ -302,8 +319,9 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
                                                        const uint32_t (&offA)[TileLanes<Cfg>::NJA],
                                                        const uint16_t* const (&baseB)[TileLanes<Cfg>::NJB],
                                                        const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
-                                                       uint8_t* lds, f32x16_t (&acc)[Cfg::TM][Cfg::TN],
+                                                       uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN],
                                                        const KMajorB& kb = KMajorB()) {
+  static_assert(!Cfg::MFMA16, "16x16x32 tiles run gemm_mainloop_fixed16");
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
   constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
@@ -642,6 +660,182 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
 #endif
 }
 
+// =============================================================================================
+// Direct path of the 256-row tiles: the same two stages of 64-element slabs, accumulated with
+// v_mfma_f32_16x16x32_bf16 in a schedule written out in source order (every MFMA fenced by scheduling
+// barriers), because with one or two wavefronts per SIMD nothing else hides a wait, and an instruction
+// that cannot issue - a load while the address unit's queue is full - holds back the MFMAs behind it.
+//  * A slab is two K steps of 32.  A step runs its TM x TN MFMAs row group by row group: the token
+//    fragment of a group (16 rows x 32 K) is single-buffered and re-read in place for the next step as
+//    soon as the group's last MFMA has issued (a whole step ahead of its next use); the TN weight
+//    fragments are double-buffered and read behind the first MFMAs of the previous step.
+//  * One barrier per slab, behind the first two row groups of the slab's second step: by then every
+//    fragment read of the stage has returned (the last one was issued two groups earlier) and the next
+//    slab, whose last loads went out more than half a slab before, has landed.
+//  * The global->LDS loads go out at the rate the address unit takes them, one 1 KB load per wave
+//    behind every fourth MFMA (16 cycles per load and CU), not in a burst behind the barrier: the
+//    first loads of the slab after next through the rest of the second step, the others during the
+//    first step of the following slab - at least half a slab ahead of the barrier that waits for them.
+// =============================================================================================
+template <class Cfg>
+__device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
+                                                      const uint16_t* const (&baseA)[TileLanes<Cfg>::NJA],
+                                                      const uint32_t (&offA)[TileLanes<Cfg>::NJA],
+                                                      const uint16_t* const (&baseB)[TileLanes<Cfg>::NJB],
+                                                      const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
+                                                      uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN]) {
+  static_assert(Cfg::MFMA16 && Cfg::DIRECT && !Cfg::B_KMAJOR, "16x16x32 schedule of the direct 256-row tiles");
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
+  constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
+  constexpr int L = NJA + NJB;
+  constexpr int STAGE = Cfg::STAGE_BYTES, A_BYTES = Cfg::A_BYTES;
+  constexpr int NM = TM * TN;
+  constexpr int BAR = 2 * TN;            // MFMAs of a slab's second step ahead of the barrier (two row groups)
+  constexpr int LEV = 4;                 // one load behind every fourth MFMA
+  constexpr int L1 = (NM - BAR) / LEV;   // loads of the slab after next that go out in the second step
+  static_assert(TM >= 3 && L1 >= 1 && L1 <= L && (L - L1) * LEV <= NM, "schedule does not fit this wave tile");
+  const int wave = tl.wave_s;
+
+  auto wave_uniform = [](const uint16_t* p) {
+    if (!Cfg::DUAL) return reinterpret_cast<void*>(const_cast<uint16_t*>(p));
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+  };
+  __amdgpu_buffer_rsrc_t rsA[NJA], rsB[NJB];
+#pragma unroll
+  for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseA[j]), 0, 0xffffffff, 0x00020000);
+#pragma unroll
+  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
+
+  // Fragment of K step s: tile row lr, logical 16-byte chunks 4 s + lh (lh = 0..3: 8 K elements each).
+  uint32_t koff[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) koff[s] = lds_swizzle(tl.lr, 4 * s + tl.lh);
+  const uint32_t a_base = (uint32_t)(tl.wm * Cfg::WTM) * kRowBytes;
+  uint32_t b_base[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) b_base[tn] = A_BYTES + (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
+
+  zero_acc<Cfg>(acc);
+  const int nk = k_len / kBK;
+
+  bf16x8_t fa[TM], fb[2][TN];
+  auto read_a = [&](int i, int stage, int ks) {
+    fa[i] = *reinterpret_cast<const bf16x8_t*>(lds + stage * STAGE + a_base + i * 16 * kRowBytes + koff[ks]);
+  };
+  auto read_b = [&](int buf, int j, int stage, int ks) {
+    fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(lds + stage * STAGE + b_base[j] + koff[ks]);
+  };
+  // Load l of a slab: the weight panel's first, then the token panel's.
+  auto load = [&](int l, int stage, int kt) {
+    uint8_t* st = lds + stage * STAGE;
+    const int ko = kt * kRowBytes;
+    if (l < NJB)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l - NJB], FFNK_LDS_PTR(st + ((l - NJB) * NWAVES + wave) * 1024), 16,
+                                               offA[l - NJB], ko, 0, 0);
+  };
+  // Four-wave tiles hold 256 accumulator registers per lane, which only fit the accumulation half of the
+  // register file.  Left to the builtin, the compiler keeps part of them in ordinary registers and moves
+  // them back and forth inside the loop (v_accvgpr_read/write around every other MFMA); the asm form
+  // pins each accumulator tile to the accumulation registers for the whole loop.
+  constexpr bool kAccPinned = NWAVES == 4;
+  auto mfma = [&](int buf, int m) {
+    const int i = m / TN, j = m % TN;
+    if constexpr (kAccPinned)
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[buf][j]), "v"(fa[i]));
+    else
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[buf][j], fa[i], acc[i][j], 0, 0, 0);
+  };
+  // First K step of slab kt (stage u): behind its MFMAs the fragments of the second step, and the last
+  // loads of slab kt + 1.
+  auto step0 = [&](int u, int kt, bool next) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      mfma(0, m);
+      __builtin_amdgcn_sched_barrier(0);
+      if (m < TN) read_b(1, m, u, 1);
+      if (m % TN == TN - 1) read_a(m / TN, u, 1);
+      if (m % LEV == LEV - 1 && L1 + m / LEV < L && next) load(L1 + m / LEV, u ^ 1, kt + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // Second K step: two row groups, the barrier, then behind the MFMAs the first-step fragments of slab
+  // kt + 1 (other stage) and the first loads of slab kt + 2 into this stage.
+  auto step1 = [&](int u, int kt, bool next, bool next2) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      if (m == BAR) {
+        dma_wait_barrier<0>();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mfma(1, m);
+      __builtin_amdgcn_sched_barrier(0);
+      if (next) {
+        if (m >= BAR && m < BAR + BAR / TN) read_a(m - BAR, u ^ 1, 0);  // the groups that ran ahead of the barrier
+        else if (m >= BAR + BAR / TN && m < BAR + BAR / TN + TN) read_b(0, m - BAR - BAR / TN, u ^ 1, 0);
+        if (m > BAR + BAR / TN && m % TN == TN - 1) read_a(m / TN, u ^ 1, 0);
+      }
+      if (m >= BAR && (m - BAR) % LEV == LEV - 1 && (m - BAR) / LEV < L1 && next2) load((m - BAR) / LEV, u, kt + 2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // Head of the tile: slab 0 whole and the first loads of slab 1, as the steady schedule leaves them.
+#pragma unroll
+  for (int l = 0; l < L; ++l) load(l, 0, 0);
+  if (nk > 1) {
+#pragma unroll
+    for (int l = 0; l < L1; ++l) load(l, 1, 1);
+    dma_wait_barrier<L1>();
+  } else {
+    dma_wait_barrier<0>();
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) read_b(0, j, 0, 0);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) read_a(i, 0, 0);
+
+  int k0 = 0;
+  for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches
+    step0(0, k0, true);
+    step1(0, k0, true, true);
+    step0(1, k0 + 1, true);
+    step1(1, k0 + 1, true, true);
+  }
+  for (; k0 < nk; k0 += 2) {
+    step0(0, k0, k0 + 1 < nk);
+    step1(0, k0, k0 + 1 < nk, k0 + 2 < nk);
+    if (k0 + 1 < nk) {
+      step0(1, k0 + 1, k0 + 2 < nk);
+      step1(1, k0 + 1, k0 + 2 < nk, k0 + 3 < nk);
+    }
+  }
+  // The compiler does not see that the asm statements are matrix instructions: give the last of them the
+  // wait states a read of its result by an ordinary instruction needs.
+  if constexpr (kAccPinned) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#endif
+}
+
+// Main loop of a direct-path tile, by the tile's MFMA shape.
+template <class Cfg>
+__device__ __forceinline__ void gemm_mainloop_direct(const TileLanes<Cfg>& tl,
+                                                     const uint16_t* const (&baseA)[TileLanes<Cfg>::NJA],
+                                                     const uint32_t (&offA)[TileLanes<Cfg>::NJA],
+                                                     const uint16_t* const (&baseB)[TileLanes<Cfg>::NJB],
+                                                     const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
+                                                     uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN],
+                                                     const KMajorB& kb = KMajorB()) {
+  if constexpr (Cfg::MFMA16) gemm_mainloop_fixed16<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc);
+  else gemm_mainloop_slab_dma<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
+}
+
 // Map a launch-order workgroup id to a position L in the tile order such that every XCD
 // (workgroup b runs on XCD b % 8) owns one contiguous range of the order: tiles that share
 // A rows / B columns then meet in the same L2.  Returns -1 for a surplus workgroup.
@@ -654,24 +848,24 @@ __device__ __forceinline__ int xcd_tile_slot(int total) {
   return L < total ? L : -1;
 }
 
-// Epilogue shared by the routed kernels.  Per 32x32 accumulator tile a lane holds token row
-// (lane & 31) and output columns 8 * (v / 4) + 4 * (lane >> 5) + (v % 4).
+// Epilogue shared by the routed kernels.  Per accumulator tile a lane holds token row lr and the output
+// columns acc_col(v, lh), i.e. runs of four consecutive columns (one 8-byte store each).
 template <class Cfg>
-__device__ __forceinline__ void routed_epilogue(const GemmArgs& g, f32x16_t (&acc)[Cfg::TM][Cfg::TN], int row0,
+__device__ __forceinline__ void routed_epilogue(const GemmArgs& g, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN], int row0,
                                                 int row_end, int n0, int wm, int wn, uint32_t lr, uint32_t lh) {
-  constexpr int TM = Cfg::TM, TN_OUT = Cfg::TN_OUT;
+  constexpr int TM = Cfg::TM, TN_OUT = Cfg::TN_OUT, MT = Cfg::MT, RUNS = Cfg::ACC_N / 4;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int p = row0 + wm * Cfg::WTM + i * 32 + (int)lr;
+    const int p = row0 + wm * Cfg::WTM + i * MT + (int)lr;
     if (p >= row_end) continue;
     const int64_t dst = Cfg::SCATTER_C ? (int64_t)g.perm[p] : (int64_t)p;
     uint16_t* crow = g.C + dst * g.ldc;
 #pragma unroll
     for (int j = 0; j < TN_OUT; ++j) {
-      const int nb = n0 + wn * Cfg::WTN_OUT + j * 32 + 4 * (int)lh;
+      const int nb = n0 + wn * Cfg::WTN_OUT + j * MT;
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int n = nb + 8 * q4;
+      for (int q4 = 0; q4 < RUNS; ++q4) {
+        const int n = nb + acc_col<Cfg>(4 * q4, (int)lh);
         float o[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -692,7 +886,7 @@ __device__ __forceinline__ void routed_epilogue(const GemmArgs& g, f32x16_t (&ac
           uint16_t* prow = g.C_pre + dst * g.ldc_pre + n;
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
-            const f32x16_t& t = acc[i][j + half * TN_OUT];
+            const typename Cfg::Acc& t = acc[i][j + half * TN_OUT];
             uint16_t* pp = prow + (int64_t)half * g.N;
             if (n + 3 < g.N && ((reinterpret_cast<uintptr_t>(pp) & 7) == 0)) {
               uint2 v2;
@@ -715,18 +909,19 @@ __device__ __forceinline__ void routed_epilogue(const GemmArgs& g, f32x16_t (&ac
 // goes to base[p * ld + n].
 template <class Cfg>
 __device__ __forceinline__ void routed_partial_store(float* base, int64_t ld, const GemmArgs& g,
-                                                     f32x16_t (&acc)[Cfg::TM][Cfg::TN], int row0, int row_end, int n0,
+                                                     typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN], int row0, int row_end, int n0,
                                                      int wm, int wn, uint32_t lr, uint32_t lh) {
+  constexpr int MT = Cfg::MT, RUNS = Cfg::ACC_N / 4;
 #pragma unroll
   for (int i = 0; i < Cfg::TM; ++i) {
-    const int p = row0 + wm * Cfg::WTM + i * 32 + (int)lr;
+    const int p = row0 + wm * Cfg::WTM + i * MT + (int)lr;
     if (p >= row_end) continue;
     float* prow = base + (int64_t)p * ld;
 #pragma unroll
     for (int j = 0; j < Cfg::TN; ++j) {
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int n = n0 + wn * Cfg::WTN_OUT + j * 32 + 8 * q4 + 4 * (int)lh;
+      for (int q4 = 0; q4 < RUNS; ++q4) {
+        const int n = n0 + wn * Cfg::WTN_OUT + j * MT + acc_col<Cfg>(4 * q4, (int)lh);
         if (n + 3 < g.N) {
           *reinterpret_cast<float4*>(prow + n) =
               make_float4(acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]);
@@ -791,8 +986,8 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   const int n0 = tc.n0 + sub_n * Cfg::BN_OUT;
   if (row0 >= row_end || n0 >= g.N) return;  // a sub-tile past the edge of a partial macro tile
 
-  f32x16_t acc[TM][TN];
-  if (Cfg::DIRECT) {
+  typename Cfg::Acc acc[TM][TN];
+  if constexpr (Cfg::DIRECT) {
     constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
     TileLanes<Cfg> rl;
     rl.init();
@@ -843,7 +1038,7 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
         offB[j] = (uint32_t)(((int64_t)(n - n_first) * g.ldb + rl.c_log * 8) * 2);
       }
     }
-    if (k_len > 0) gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
+    if (k_len > 0) gemm_mainloop_direct<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
     else zero_acc<Cfg>(acc);  // a range past the end of K contributes exact zeros
     if (!Cfg::DUAL && splits > 1) {
       if (g.tail_mode == 3)  // one compact fp32 tile per (tile, range) pair
@@ -919,7 +1114,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
   TileLanes<Cfg> rl;
   rl.init();
   const int r0 = tile_r * BN, c0 = tile_c * BM;
-  f32x16_t acc[TM][TN];
+  typename Cfg::Acc acc[TM][TN];
   if (k_len > 0) {
     const uint16_t* baseA[NJA];
     uint32_t offA[NJA];
@@ -956,25 +1151,26 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
         offB[j] = (uint32_t)(((int64_t)(r - r_first) * g.lda + rl.c_log * 8) * 2);
       }
     }
-    gemm_mainloop_slab_dma<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
+    gemm_mainloop_direct<Cfg>(rl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
   } else {
     zero_acc<Cfg>(acc);  // a split without slabs (e.g. an empty modality) contributes exact zeros
   }
 
-  // acc[i][j][v]: BM-panel row (= output column c) c0 + wm*WTM + i*32 + (lane&31);
-  //               BN-panel row (= output row r) r0 + wn*WTN + j*32 + 8*(v/4) + 4*(lane>>5) + v%4.
+  // acc[i][j][v]: BM-panel row (= output column c) c0 + wm*WTM + i*MT + lr;
+  //               BN-panel row (= output row r) r0 + wn*WTN + j*MT + acc_col(v, lh).
+  constexpr int MT = Cfg::MT, RUNS = Cfg::ACC_N / 4;
   if (g.out[0] != nullptr) {
     // single split: the sums are complete, store bf16 with the caller's strides
     uint16_t* out = g.out[grp];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int c = c0 + rl.wm * Cfg::WTM + i * 32 + (int)rl.lr;
+      const int c = c0 + rl.wm * Cfg::WTM + i * MT + (int)rl.lr;
       if (c >= g.Cc) continue;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int r = r0 + rl.wn * Cfg::WTN_OUT + j * 32 + 8 * q4 + 4 * (int)rl.lh;
+        for (int q4 = 0; q4 < RUNS; ++q4) {
+          const int r = r0 + rl.wn * Cfg::WTN_OUT + j * MT + acc_col<Cfg>(4 * q4, (int)rl.lh);
           uint16_t* dst = out + (int64_t)r * g.out_sr + (int64_t)c * g.out_sc;
           if (g.out_sr == 1 && r + 3 < g.R && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
             uint2 v2;
@@ -984,7 +1180,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              if (r + e < g.R) dst[(int64_t)e * g.out_sr] = f2bf(acc[i][j][4 * q4 + e]);  // out_sc == 1: 32 lanes -> 64 contiguous bytes
+              if (r + e < g.R) dst[(int64_t)e * g.out_sr] = f2bf(acc[i][j][4 * q4 + e]);  // out_sc == 1: MT lanes -> 2 MT contiguous bytes
           }
         }
       }
@@ -994,14 +1190,14 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
   float* P = g.P + ((int64_t)(grp * g.splits + split)) * g.R * g.Cc;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int c = c0 + rl.wm * Cfg::WTM + i * 32 + (int)rl.lr;
+    const int c = c0 + rl.wm * Cfg::WTM + i * MT + (int)rl.lr;
     if (c >= g.Cc) continue;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int r = r0 + rl.wn * Cfg::WTN_OUT + j * 32 + 8 * (v / 4) + 4 * (int)rl.lh + (v % 4);
-        if (r < g.R) P[(int64_t)r * g.Cc + c] = acc[i][j][v];  // 32 lanes -> 32 consecutive floats
+      for (int v = 0; v < Cfg::ACC_N; ++v) {
+        const int r = r0 + rl.wn * Cfg::WTN_OUT + j * MT + acc_col<Cfg>(v, (int)rl.lh);
+        if (r < g.R) P[(int64_t)r * g.Cc + c] = acc[i][j][v];  // MT lanes -> MT consecutive floats
       }
     }
   }
