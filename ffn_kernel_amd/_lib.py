@@ -20,6 +20,7 @@ _SIGNATURES = {
     "ffnk_version": (c_int, []),
     "ffnk_last_error": (c_char_p, []),
     "ffnk_debug_force_tile": (c_int, [c_int]),
+    "ffnk_debug_force_splits": (c_int, [c_int]),
     "ffnk_route": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "ffnk_workspace_bytes": (c_size_t, [c_int, c_int64, c_int64, c_int64]),
     "ffnk_tile_config": (c_int, [c_int, c_int64, c_int64, c_int64, c_void_p]),

@@ -69,6 +69,20 @@ RouteWs carve_route(uint8_t* ws, int64_t M) {
   return r;
 }
 
+// Tuner overrides, see ffnk_debug_force_tile / ffnk_debug_force_splits.
+std::atomic<int> g_force_tile{-1};    // 0..3: that tile; -1: table, then rules; -2: rules only
+std::atomic<int> g_force_splits{-1};  // >= 1: that split-K factor where a GEMM can be split
+
+int forced_tile() {
+  const int t = g_force_tile.load(std::memory_order_relaxed);
+  return (t >= 0 && t < TILE_COUNT) ? t : -1;
+}
+bool use_tuned() { return g_force_tile.load(std::memory_order_relaxed) != -2; }
+int forced_splits() {
+  const int s = g_force_splits.load(std::memory_order_relaxed);
+  return (s >= 1 && s <= 16) ? s : -1;
+}
+
 int64_t padded_rows(int64_t M) { return round_up64(M, 64) + 64; }  // >= pad64(nv) + pad64(M - nv)
 
 struct BwdPlan {
@@ -83,7 +97,9 @@ BwdPlan plan_bwd(int64_t M, int64_t K, int64_t N, bool dw_k_contig) {
   p.dw_k_contig = dw_k_contig;
   p.R = dw_k_contig ? N : K;
   p.Cc = dw_k_contig ? K : N;
-  p.tc = pick_splitk_tile(M, p.R, p.Cc);
+  p.tc = pick_splitk_tile(M, p.R, p.Cc, use_tuned());
+  if (forced_tile() >= 0) p.tc.tile = forced_tile();
+  if (forced_splits() >= 1) p.tc.splits = forced_splits();
   p.ldt = padded_rows(M);
   size_t o = route_ws_bytes(M);
   p.off_wt = o; o += 2 * ws_align((size_t)K * N * 2);
@@ -143,13 +159,6 @@ bool kmajor_ok(int64_t K, int64_t N, int64_t ldb, const void* w0, const void* w1
          ldb * 128 + 2 * N < k4g;
 }
 
-std::atomic<int> g_force_tile{-1};  // tuner override, see ffnk_debug_force_tile
-
-int forced_tile() {
-  const int t = g_force_tile.load(std::memory_order_relaxed);
-  return (t >= 0 && t < TILE_COUNT) ? t : -1;
-}
-
 // Scratch of ffnk_masked_ffn_fwd_static: one copy per GPU, held from the moment the library's code
 // object is loaded there until the process ends.  The name is a host-side stand-in, not a device
 // address: host code only ever uses the per-device address that static_scratch() looks up.
@@ -174,9 +183,9 @@ int static_scratch(void** out) {
   return FFNK_OK;
 }
 
-int routed_tile(int64_t M, int64_t n_out, bool dual) {
+int routed_tile(int64_t M, int64_t n_out, bool dual, int64_t K = 0) {
   const int f = forced_tile();
-  return f >= 0 ? f : pick_routed_tile(M, n_out, dual);
+  return f >= 0 ? f : pick_routed_tile(M, n_out, dual, K, use_tuned());
 }
 
 bool use_stream_path(int64_t M, int64_t d, int64_t h) { return stream_shape_ok(M, d, h); }
@@ -206,8 +215,12 @@ RoutedPlan down_plan(int64_t M, int64_t d, int64_t h) {
     p.tile = f;
     p.splits = pick_routed_splits(M, d, h, p.tile);
   } else {
-    p = pick_routed_plan(M, d, h);
+    p = pick_routed_plan(M, d, h, use_tuned());
   }
+  // a forced split-K factor: whole 64-element slabs, no empty range, what the reduce pass can address
+  if (const int fs = forced_splits(); fs >= 1 && h % 64 == 0 && M < 65536 && cdiv64(h / 64, cdiv64(h / 64, fs)) == fs &&
+      p.tile != TILE_256x256_W4)
+    p.splits = fs;
   return p;
 }
 // MaskedLinear forward at decode sizes: 0 = LDS-tiled GEMM, 1 = dot-product streams (M <= 8),
@@ -257,8 +270,10 @@ extern "C" {
 int ffnk_version(void) { return FFNK_VERSION; }
 
 int ffnk_debug_force_tile(int tile) {
-  return g_force_tile.exchange((tile >= 0 && tile < TILE_COUNT) ? tile : -1);
+  return g_force_tile.exchange(((tile >= 0 && tile < TILE_COUNT) || tile == -2) ? tile : -1);
 }
+
+int ffnk_debug_force_splits(int splits) { return g_force_splits.exchange((splits >= 1 && splits <= 16) ? splits : -1); }
 
 const char* ffnk_last_error(void) { return g_err; }
 
@@ -313,12 +328,12 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   switch (op) {
     case FFNK_OP_LINEAR_FWD: { const RoutedPlan lp = linear_plan(M, K, N); tile = lp.tile; splits = lp.splits; contraction = K; break; }
     case FFNK_OP_FFN_FWD:
-    case FFNK_OP_FFN_UP: tile = pick_routed_tile(M, N, true); dual = true; contraction = K; break;
+    case FFNK_OP_FFN_UP: tile = routed_tile(M, N, true, K); dual = true; contraction = K; break;
     case FFNK_OP_FFN_DOWN: tile = down_plan(M, K, N).tile; contraction = N; break;  // out cols = d = K, contraction h = N
     case FFNK_OP_LINEAR_BWD:
-    case FFNK_OP_BWD_DX: tile = pick_routed_tile(M, K, false); contraction = N; break;
+    case FFNK_OP_BWD_DX: tile = routed_tile(M, K, false); contraction = N; break;
     case FFNK_OP_BWD_DW: {
-      const TileChoice c = pick_splitk_tile(M, N, K);
+      const TileChoice c = plan_bwd(M, K, N, true).tc;
       tile = c.tile; splits = c.splits; contraction = M; break;
     }
     default: return fail(FFNK_E_OP, "unknown op %d", op);
@@ -577,7 +592,7 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
   up.perm = r.perm; up.counts = r.counts;
   up.M = (int)M; up.N = (int)h; up.K = (int)d;
   up.C_pre = pre; up.ldc_pre = pre_stride_m;
-  FFNK_HIP(launch_up_gemm(routed_tile(M, h, true), direct_ok(d, M, x_stride_m, up_stride_n), up, stream), "up-projection GEMM");
+  FFNK_HIP(launch_up_gemm(routed_tile(M, h, true, d), direct_ok(d, M, x_stride_m, up_stride_n), up, stream), "up-projection GEMM");
   FFNK_HIP(mark(1), "event record");
   GemmArgs dn;
   dn.A = H; dn.lda = ldh;
@@ -861,7 +876,8 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   if (in_place) {
     FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, x, x_stride_m, (int)d, XT, p.ldt, r.perm, r.counts, (int)M,
                                       stream, false, false), "g / x transpose");
-    const TileChoice tc = pick_splitk_tile(M, h, d);
+    TileChoice tc = pick_splitk_tile(M, h, d, use_tuned());
+    if (forced_splits() >= 1) tc.splits = forced_splits();
     const int tile = forced_tile() >= 0 ? forced_tile() : tc.tile;
     // out[r * sr + c * sc]: r runs over h (the in-place operand's columns), c over d
     auto weight_grad_in_place = [&](const uint16_t* rows, int64_t ld_rows, const uint16_t* cT, uint16_t* o0, uint16_t* o1,

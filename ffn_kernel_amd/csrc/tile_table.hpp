@@ -22,8 +22,37 @@ struct TileChoice {
   int splits;  // split-K factor (weight-gradient GEMM only)
 };
 
-// Routed GEMM over M rows and n_out output columns.
-inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual) {
+// Measured plans.  `python -m ffn_kernel_amd.tune --emit` times every candidate (tile x split-K factor)
+// per operation, shape and M bucket on the GPU and writes tile_table_gen.hpp: one entry wherever the best
+// candidate beat the rules and the cost model below by a margin.  The pick_* functions consult these
+// entries first (exact contraction / output extents, M inside the bucket) and fall back to the rules.
+// This is what the reference's find_spec/*.py searches and bf16_*.json tables are to its kernels
+// (find_spec/find.py:18-64, ffn_kernel/utils.py:3-5).
+enum TunedOp : int {
+  TUNED_PLAIN = 0,   // single-weight routed GEMM: k = contraction, n = output columns
+  TUNED_DUAL = 1,    // SwiGLU GEMM: k = contraction (d), n = output columns (h)
+  TUNED_SPLITK = 2,  // weight-gradient GEMM: k = R (rows of the in-place operand), n = Cc
+};
+struct TunedPlan {
+  int op;            // TunedOp, -1 ends the table
+  int m_lo, m_hi;    // rows M of the call, inclusive
+  int k, n;
+  int tile, splits;
+};
+}  // namespace ffnk
+#include "tile_table_gen.hpp"
+namespace ffnk {
+
+inline const TunedPlan* tuned_plan(int op, int64_t M, int64_t k, int64_t n) {
+  for (const TunedPlan* p = kTunedPlans; p->op >= 0; ++p)
+    if (p->op == op && p->k == k && p->n == n && M >= p->m_lo && M <= p->m_hi) return p;
+  return nullptr;
+}
+
+// Routed GEMM over M rows and n_out output columns (K: the contraction, 0 = not known to the caller).
+inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual, int64_t K = 0, bool use_table = true) {
+  if (use_table && dual && K > 0)
+    if (const TunedPlan* t = tuned_plan(TUNED_DUAL, M, K, n_out)) return t->tile;
   auto tiles = [&](int tile) {
     const TileGeom t = tile_geom(tile, dual);
     return cdiv64(M, t.block_m) * cdiv64(n_out, t.block_n_out);
@@ -90,8 +119,14 @@ inline int pick_routed_splits(int64_t M, int64_t n_out, int64_t K, int tile) {
   return best;
 }
 
-inline RoutedPlan pick_routed_plan(int64_t M, int64_t n_out, int64_t K) {
+inline RoutedPlan pick_routed_plan(int64_t M, int64_t n_out, int64_t K, bool use_table = true) {
   RoutedPlan p;
+  if (use_table)
+    if (const TunedPlan* t = tuned_plan(TUNED_PLAIN, M, K, n_out)) {
+      p.tile = t->tile;
+      p.splits = (K % 64 == 0 && M < 65536 && n_out % 4 == 0) ? t->splits : 1;
+      return p;
+    }
   p.tile = pick_routed_tile(M, n_out, false);
   p.splits = 1;
   if (M > 4096 || K % 64 != 0) return p;
@@ -110,8 +145,14 @@ inline RoutedPlan pick_routed_plan(int64_t M, int64_t n_out, int64_t K) {
 }
 
 // Weight-gradient GEMM: two [R, Cc] outputs, contraction over about M / 2 rows each.
-inline TileChoice pick_splitk_tile(int64_t M, int64_t R, int64_t Cc) {
+inline TileChoice pick_splitk_tile(int64_t M, int64_t R, int64_t Cc, bool use_table = true) {
   TileChoice c;
+  if (use_table)
+    if (const TunedPlan* t = tuned_plan(TUNED_SPLITK, M, R, Cc)) {
+      c.tile = t->tile;
+      c.splits = t->splits;
+      return c;
+    }
   // Large outputs: the 256x256 tile fills the chip on its own, no split needed (and the GEMM then
   // stores bf16 directly, without partials or a reduce pass).
   if (2 * cdiv64(R, 256) * cdiv64(Cc, 256) >= 2 * kCus) {

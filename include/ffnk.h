@@ -101,14 +101,19 @@ FFNK_API size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N);
 FFNK_API int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t* out);
 
 /*
- * Tuner-only hook: force every LDS-tiled GEMM launched by this process to use tile id `tile`
- * (0 = 256x256 / 8 waves, 1 = 256x256 / 4 waves, 2 = 128x128 / 4 waves, 3 = small), or -1 to
- * return to the tile table.  The one piece of process-global state in the library (an atomic int
- * read at every launch): it exists for the tuner (python -m ffn_kernel_amd.tune, the counterpart of
- * the reference's find_spec/*.py sweeps) and for tests that run every compiled tile; production
- * callers leave it alone.  Returns the previous value.
+ * Tuner-only hooks (python -m ffn_kernel_amd.tune, the counterpart of the reference's find_spec/*.py
+ * sweeps, and the tests that run every compiled tile).  ffnk_debug_force_tile: every LDS-tiled GEMM
+ * launched by this process uses tile id `tile` (0 = 256x256 / 8 waves, 1 = 256x256 / 4 waves,
+ * 2 = 128x128 / 4 waves, 3 = small); -1 returns to the tile table (measured plans first, then the
+ * rules); -2 uses the rules only, ignoring the measured plans (what the tuner compares against).
+ * ffnk_debug_force_splits: every GEMM that can cut its contraction (single-weight routed GEMMs with
+ * a workspace, weight-gradient GEMMs) uses `splits` ranges (1..16) where the shape allows it; -1
+ * returns to the table.  Both are process-global atomics read at every call (ffnk_workspace_bytes
+ * answers for the current setting); production callers leave them alone.  Each returns the previous
+ * value.
  */
 FFNK_API int ffnk_debug_force_tile(int tile);
+FFNK_API int ffnk_debug_force_splits(int splits);
 
 /*
  * MaskedLinear forward — replaces _bf16_linear_forward (ffn_kernel/linear.py:418-452):

@@ -189,3 +189,38 @@ def test_row_limit_is_what_one_route_launch_handles():
     assert _lib.workspace_bytes(_lib.OP_LINEAR_FWD, 1 << 22, 64, 64) > 0
     with pytest.raises(ValueError):
         _lib.workspace_bytes(_lib.OP_LINEAR_FWD, (1 << 22) + 1, 64, 64)
+
+
+def test_measured_plans_are_consulted_before_the_rules():
+    """Every entry of the generated table is what ffnk_tile_config reports for a shape inside its bucket,
+    ffnk_debug_force_tile(-2) falls back to the rules, and the tuner's renderer reproduces the committed
+    file byte for byte from its own entries."""
+    from ffn_kernel_amd import tune
+    text = tune.GEN_PATH.read_text()
+    entries = [tuple(map(int, e)) for e in re.findall(r"^\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},$", text, re.M)]
+    assert tune.render_header(entries) == text
+    geom = {0: (256, 256, 8), 1: (256, 256, 4), 2: (128, 128, 4)}
+    lib = _lib.load()
+    checked = 0
+    for op, lo, hi, k, n, tile, splits in entries:
+        if op == tune.TUNED_DUAL:
+            cfg = _lib.tile_config(_lib.OP_FFN_UP, hi, k, n)
+            if tile in geom:
+                assert (cfg["block_m"], cfg["waves_m"] * cfg["waves_n"]) == (geom[tile][0], geom[tile][2]), (op, hi, k, n, cfg)
+            checked += 1
+        elif op == tune.TUNED_PLAIN:
+            cfg = _lib.tile_config(_lib.OP_FFN_DOWN, hi, n, k)  # FFN extents: K = d = output columns, N = h = contraction
+            if cfg["path"] == _lib.PATH_MFMA_TILED:
+                assert cfg["split_k"] == splits, (op, hi, k, n, cfg)
+                if tile in geom:
+                    assert (cfg["block_m"], cfg["block_n"]) == geom[tile][:2]
+                checked += 1
+    assert checked > 0 or not entries
+    if entries:
+        op, lo, hi, k, n, tile, splits = next((e for e in entries if e[0] == tune.TUNED_PLAIN), entries[0])
+        try:
+            assert lib.ffnk_debug_force_tile(-2) == -1
+            rules = _lib.tile_config(_lib.OP_FFN_DOWN, hi, n, k)
+        finally:
+            lib.ffnk_debug_force_tile(-1)
+        assert isinstance(rules["split_k"], int)

@@ -1,0 +1,73 @@
+"""The user-facing tools on the GPU: the check CLI (the non-interactive counterpart of the reference's
+test_linear.py / test_ffn.py --check flows) and the tuner that produces the measured tile table."""
+import json
+import re
+
+import pytest
+import torch
+
+from ffn_kernel_amd import _lib, check, tune
+
+from helpers import note
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("argv", [
+    ["linear", "--check", "--max-mult", "2"],
+    ["linear", "--check", "--bsz", "2", "--max-mult", "1", "--d", "512"],
+    ["ffn", "--check", "--max-mult", "2"],
+    ["ffn", "--check", "--bwd", "--max-mult", "1", "--d", "512", "--h", "1024"],
+])
+def test_check_cli_passes(dev, argv, capsys):
+    note(f"check CLI {' '.join(argv)}")
+    assert check.main(argv) == 0
+    lines = [json.loads(l) for l in capsys.readouterr().out.splitlines() if l.startswith("{")]
+    assert lines and all(l["ok"] for l in lines)
+    assert all(k.startswith("rel_l2") and v <= 2e-2 for l in lines for k, v in l.items() if k.startswith("rel_l2"))
+
+
+def test_check_cli_times_both_modules(dev, capsys):
+    note("check CLI timing mode")
+    assert check.main(["ffn", "--max-mult", "1"]) == 0
+    rec = json.loads([l for l in capsys.readouterr().out.splitlines() if l.startswith("{")][-1])
+    assert rec["pytorch_ms"] > 0 and rec["hip_ms"] > 0
+
+
+def test_tuner_emits_a_table_the_library_can_compile(dev, tmp_path, capsys):
+    """A short sweep (two M buckets per layer) through every candidate, forced via the C ABI; the
+    emitted header has the generated file's format, and the overrides are back to the table after it."""
+    note("tuner --quick --emit")
+    out = tmp_path / "tile_table_gen.hpp"
+    assert tune.main(["--quick", "--trials", "2", "--emit", "--out", str(out), "--json", str(tmp_path / "t.json")]) == 0
+    text = out.read_text()
+    entries = re.findall(r"^\s*\{(-?\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},$", text, re.M)
+    assert entries and entries[-1][0] == "-1"
+    for op, lo, hi, k, n, tile, splits in entries[:-1]:
+        assert int(op) in (0, 1, 2) and int(lo) <= int(hi) and 0 <= int(tile) <= 3 and 1 <= int(splits) <= 16
+    recs = json.loads((tmp_path / "t.json").read_text())
+    assert {r["op"] for r in recs} == {"ffn_fwd", "linear_fwd", "linear_bwd"}
+    lib = _lib.load()
+    assert lib.ffnk_debug_force_tile(-1) == -1 and lib.ffnk_debug_force_splits(-1) == -1
+
+
+def test_forced_splits_results_match(dev):
+    """A forced split-K factor changes the summation order only: results stay within bf16 of the unsplit ones."""
+    note("forced splits: linear fwd M=300 K=2048 N=512")
+    from ffn_kernel_amd import MaskedLinear
+    from ffn_kernel_amd import workloads as wl
+    from oracle import cref
+    from helpers import assert_close
+    M, K, N = 300, 2048, 512
+    mask = torch.rand(M, generator=torch.Generator().manual_seed(3)) < 0.5
+    w = wl.make_linear("t", M, K, N, mask, seed=5, w_std=0.05)
+    dw = w.to(dev)
+    ref = cref.linear_fwd(w.x, w.Wv, w.Wt, w.mask)
+    lib = _lib.load()
+    try:
+        for s in (1, 2, 4):
+            lib.ffnk_debug_force_splits(s)
+            assert _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, N)["split_k"] == s
+            assert_close(MaskedLinear.apply(dw.x, dw.Wv.T, dw.Wt.T, dw.mask), ref, f"splits {s}")
+    finally:
+        lib.ffnk_debug_force_splits(-1)
