@@ -263,6 +263,37 @@ size_t tiled_down_partial_bytes(int64_t M, int64_t d, int64_t h) {
   return 0;
 }
 
+// Split-K factor of the weight-gradient GEMM when it shares a launch with the dx GEMM (both on 128x128
+// tiles, two workgroups per CU).  The weight-gradient workgroups are few and long, the dx workgroups many
+// and short and fill the CUs the others leave: the launch lasts as long as the longer of the two, in
+// 64-row slabs of 0.8 us (a 128x128 tile's slab behind two LDS stages waits on its loads: measured).  Unsplit (no partials, no reduce pass, one launch fewer) unless cutting the
+// contraction shortens the estimate by more than 40 % (at M = 8192, K = N = 1024 two ranges measure 7 % slower than one); never more ranges than the plan sized
+// the partials for.
+int fused_bwd_splits(int64_t M, int64_t K, int64_t N, int plan_splits) {
+  if (forced_splits() >= 1) return plan_splits;  // the tuner's factor went into the plan
+  const double slots = 2.0 * kCus, t_slab = 0.8;
+  const double dw_tiles = 2.0 * (double)cdiv64(N, 128) * (double)cdiv64(K, 128);
+  const double dx_units = (double)(cdiv64(M, 128) + 1) * (double)cdiv64(K, 128) * (double)cdiv64(N, 64);
+  auto estimate = [&](int s) {
+    const double dw_wgs = dw_tiles * s;
+    const double dw_slabs = (double)cdiv64(cdiv64(M, 2 * 64), s) * (double)cdiv64((int64_t)dw_wgs, (int64_t)slots);
+    const double rest = slots - dw_wgs > slots / 8 ? slots - dw_wgs : slots / 8;
+    const double t = (dw_slabs > dx_units / rest ? dw_slabs : dx_units / rest) * t_slab;
+    return s == 1 ? t : t + 4.0 + (double)s * 2.0 * (double)K * (double)N * 8.0 / 4.0e6;  // launch + partials at 4 TB/s
+  };
+  const double unsplit = estimate(1);
+  int best = 1;
+  double best_t = unsplit;
+  for (int s = 2; s <= plan_splits; ++s) {
+    const double t = estimate(s);
+    if (t < best_t) {
+      best = s;
+      best_t = t;
+    }
+  }
+  return best_t < 0.6 * unsplit ? best : 1;
+}
+
 }  // namespace
 
 extern "C" {
@@ -347,7 +378,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->waves_m = gm.waves_m;
   out->waves_n = gm.waves_n;
   out->lds_stages = 2;
-  out->group_m = 8;
+  out->group_m = dual ? 8 : 4;
   out->split_k = splits;
   out->direct_lds = (contraction > 0 && contraction % 64 == 0) ? 1 : 0;
   if (op == FFNK_OP_FFN_DOWN && !stream) out->split_k = tiled_down_splits(M, K, N);
@@ -720,8 +751,14 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   a.C = dx; a.ldc = dx_stride_m;
   a.perm = r.perm; a.counts = r.counts;
   a.M = (int)M; a.N = (int)K; a.K = (int)N;
-  if (w_kmajor) FFNK_HIP(launch_linear_gemm_kmajor(routed_tile(M, K, false), a, stream), "dx GEMM");
-  else FFNK_HIP(launch_linear_gemm(routed_tile(M, K, false), direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
+  const int dx_tile = routed_tile(M, K, false);
+  // Both GEMMs on the 128x128 tile and the weights readable in place: one launch runs the two side by
+  // side (after the transposes it depends on), see below.
+  const bool fused = w_kmajor && dx_tile == TILE_128x128_W4 && p.tc.tile == TILE_128x128_W4;
+  if (!fused) {
+    if (w_kmajor) FFNK_HIP(launch_linear_gemm_kmajor(dx_tile, a, stream), "dx GEMM");
+    else FFNK_HIP(launch_linear_gemm(dx_tile, direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
+  }
 
   // ---- dW_g = x_g^T g_g, contraction over the rows of group g ----
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]
@@ -736,10 +773,12 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   s.R = (int)p.R; s.Cc = (int)p.Cc; s.splits = p.tc.splits;
   const int64_t sr = p.dw_k_contig ? dw_stride_n : dw_stride_k;
   const int64_t sc = p.dw_k_contig ? dw_stride_k : dw_stride_n;
-  if (p.tc.splits == 1) { s.out[0] = dWv; s.out[1] = dWt; s.out_sr = sr; s.out_sc = sc; }
-  FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
-  if (p.tc.splits > 1)
-    FFNK_HIP(launch_splitk_reduce(P, p.tc.splits, (int)p.R, (int)p.Cc, dWv, dWt, sr, sc, stream), "dW reduce");
+  if (fused) s.splits = fused_bwd_splits(M, K, N, p.tc.splits);
+  if (s.splits == 1) { s.out[0] = dWv; s.out[1] = dWt; s.out_sr = sr; s.out_sc = sc; }
+  if (fused) FFNK_HIP(launch_fused_bwd(a, s, stream), "fused dx / dW GEMM");
+  else FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
+  if (s.splits > 1)
+    FFNK_HIP(launch_splitk_reduce(P, s.splits, (int)p.R, (int)p.Cc, dWv, dWt, sr, sc, stream), "dW reduce");
   return FFNK_OK;
 }
 

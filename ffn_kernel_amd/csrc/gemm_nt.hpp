@@ -840,11 +840,11 @@ __device__ __forceinline__ void gemm_mainloop_direct(const TileLanes<Cfg>& tl,
 // (workgroup b runs on XCD b % 8) owns one contiguous range of the order: tiles that share
 // A rows / B columns then meet in the same L2.  Returns -1 for a surplus workgroup.
 
-__device__ __forceinline__ int xcd_tile_slot(int total) {
+__device__ __forceinline__ int xcd_tile_slot(int total, int bid) {
   const int per_xcd = cdiv(total, kXcds);
-  const int slot = blockIdx.x / kXcds;
+  const int slot = bid / kXcds;
   if (slot >= per_xcd) return -1;
-  const int L = (blockIdx.x % kXcds) * per_xcd + slot;
+  const int L = (bid % kXcds) * per_xcd + slot;
   return L < total ? L : -1;
 }
 
@@ -939,12 +939,12 @@ __device__ __forceinline__ void routed_partial_store(float* base, int64_t ld, co
 //   GATHER_A : A row of routed position p is perm[p] (else p)
 //   SCATTER_C: C row of routed position p is perm[p] (else p)
 //   DUAL     : C = silu(A B0^T) * (A B1^T)   (SwiGLU epilogue in fp32 registers)
+// `bid`: the workgroup's index among those of this GEMM (the launch's block index, or its offset inside a
+// launch that runs several GEMMs side by side); `lds`: Cfg::LDS_BYTES, 1 KB aligned.
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) {
+__device__ __forceinline__ void routed_gemm_body(const GemmArgs& g, uint8_t* lds, const int bid) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
-
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[Cfg::LDS_BYTES];
 
   // ---- tile schedule (all from device-side counts; no host sync) ----
   const int SBM = g.sched_bm > 0 ? g.sched_bm : BM;
@@ -954,7 +954,7 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   int L, sub_m = 0, sub_n = 0, split = 0, splits = 1, tail_slot = 0;
   if (g.tail_mode == 0) {
     splits = g.splits;
-    L = xcd_tile_slot(total * splits);
+    L = xcd_tile_slot(total * splits, bid);
     if (splits > 1 && L >= 0) {  // range-major: neighbours in the order share panels, not a K range
       split = L / total;
       L -= split * total;
@@ -962,17 +962,17 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   } else {
     const int full = total / kCusPerChip * kCusPerChip;
     if (g.tail_mode == 1) {
-      L = xcd_tile_slot(full);
+      L = xcd_tile_slot(full, bid);
     } else if (g.tail_mode == 2) {
       const int qn = SBN / Cfg::BN_OUT, q = (SBM / BM) * qn;  // own tiles per macro tile
-      if ((int)blockIdx.x >= (total - full) * q) return;
-      L = full + (int)blockIdx.x / q;
-      sub_m = ((int)blockIdx.x % q) / qn;
-      sub_n = ((int)blockIdx.x % q) % qn;
+      if (bid >= (total - full) * q) return;
+      L = full + bid / q;
+      sub_m = (bid % q) / qn;
+      sub_n = (bid % q) % qn;
     } else {
       const int n_tail = total - full;
       splits = tail_split_factor(n_tail, g.K / kBK);
-      tail_slot = (int)blockIdx.x;
+      tail_slot = bid;
       if (tail_slot >= n_tail * splits) return;
       split = tail_slot / n_tail;
       L = full + tail_slot % n_tail;
@@ -1074,17 +1074,21 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   }
 }
 
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[Cfg::LDS_BYTES];
+  routed_gemm_body<Cfg>(g, lds, (int)blockIdx.x);
+}
+
 // Grouped split-K GEMM of the weight gradients (operands are padded to 64-element slabs, so
 // the direct path always applies).  With Cfg::B_KMAJOR the operand A is not a padded transpose but
 // the original [rows, R] matrix in routed order (see SplitKArgs).
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArgs g) {
+__device__ __forceinline__ void grouped_splitk_body(const SplitKArgs& g, uint8_t* lds, const int bid) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
   constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
   static_assert(!Cfg::DUAL && Cfg::DIRECT, "split-K GEMM runs on padded, 64-aligned slabs");
-
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[Cfg::LDS_BYTES];
 
   // The BM-row LDS panel holds rows of B (output columns) and the BN-row panel holds rows of A
   // (output rows): a 32-lane half wave then owns 32 consecutive output columns of one output
@@ -1092,7 +1096,7 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
   const int tiles_r = cdiv(g.R, BN);
   const int tiles_c = cdiv(g.Cc, BM);
   const int per_grp = tiles_r * tiles_c * g.splits;
-  int L = xcd_tile_slot(2 * per_grp);
+  int L = xcd_tile_slot(2 * per_grp, bid);
   if (L < 0) return;
   const int grp = L / per_grp;
   L -= grp * per_grp;
@@ -1201,6 +1205,25 @@ __global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArg
       }
     }
   }
+}
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void grouped_splitk_kernel(const SplitKArgs g) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[Cfg::LDS_BYTES];
+  grouped_splitk_body<Cfg>(g, lds, (int)blockIdx.x);
+}
+
+// The MaskedLinear backward's two GEMMs in one launch, as the reference's _fused_bwd_kernel runs dA and
+// dB by program-id range (ffn_kernel/linear.py:15-72): workgroups [0, dw_blocks) compute weight-gradient
+// tiles (the long ones: they start first), the rest dx tiles.  The two share nothing but perm / counts,
+// so the chip is filled by both at once instead of by each in turn with a partial last round.
+template <class CfgDx, class CfgDw>
+__global__ __launch_bounds__(CfgDx::NT) void fused_bwd_kernel(const GemmArgs gx, const SplitKArgs gw, const int dw_blocks) {
+  static_assert(CfgDx::NT == CfgDw::NT, "one workgroup size for both GEMMs");
+  constexpr int kLds = CfgDx::LDS_BYTES > CfgDw::LDS_BYTES ? CfgDx::LDS_BYTES : CfgDw::LDS_BYTES;
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kLds];
+  if ((int)blockIdx.x < dw_blocks) grouped_splitk_body<CfgDw>(gw, lds, (int)blockIdx.x);
+  else routed_gemm_body<CfgDx>(gx, lds, (int)blockIdx.x - dw_blocks);
 }
 
 // Upper bound on the number of workgroups the kernel needs, rounded so that every XCD gets the

@@ -5,15 +5,16 @@
 
 namespace ffnk {
 
-constexpr int kGroupM = 8;  // M-tiles per L2 super-group in the tile order (4 times the same, 16 costs 6 % at d=4096, h=14336)
+constexpr int kGroupM = 8;       // M-tiles per L2 super-group in the tile order of the SwiGLU GEMM (4: the same, 16 costs 6 % at d=4096, h=14336)
+constexpr int kGroupMPlain = 4;  // single-weight GEMMs: long contractions make wide token panels, 4 x 8 tiles per XCD round re-read fewer of them (1-2 % at K=14336)
 
 // Plain (single-weight) tiles: BN = output columns.
 template <bool GATHER, bool SCATTER, bool DIRECT>
 struct PlainTiles {
-  using T0 = RoutedGemmCfg<256, 256, 2, 4, false, GATHER, SCATTER, DIRECT, kGroupM>;
-  using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupM>;
-  using T2 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupM>;
-  using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupM>;
+  using T0 = RoutedGemmCfg<256, 256, 2, 4, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
+  using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
+  using T2 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
+  using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
 };
 
 // The same tiles over K-major weights ([K, N] rows, N contiguous; direct path only).

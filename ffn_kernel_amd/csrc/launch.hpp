@@ -45,6 +45,11 @@ hipError_t launch_splitk_gemm(int tile, const SplitKArgs& g, hipStream_t stream)
 // The same with A read in place: [rows, R] in routed order instead of a padded transpose (SplitKArgs).
 hipError_t launch_splitk_gemm_kmajor(int tile, const SplitKArgs& g, hipStream_t stream);
 
+// The MaskedLinear backward's dx GEMM (K-major weights, as launch_linear_gemm_kmajor on the 128x128 tile)
+// and its weight-gradient GEMM (as launch_splitk_gemm on the 128x128 tile) in ONE launch: weight-gradient
+// workgroups first, dx workgroups behind them.
+hipError_t launch_fused_bwd(const GemmArgs& gx, const SplitKArgs& gw, hipStream_t stream);
+
 // ---- prep.hip: layout passes around the GEMMs ----
 // dst[r, c] (row-major, ld_dst) = src[r * sr + c * sc] for r < rows, c < cols.
 hipError_t launch_strided_copy2d(const uint16_t* src, int64_t sr, int64_t sc, uint16_t* dst, int64_t ld_dst,

@@ -851,3 +851,29 @@ def test_ffn_fwd_bwd_on_unaligned_views(dev):
     assert_close(dx, rdx, "linear dx")
     assert_close(dWv.T, rdWv, "linear dWv")
     assert_close(dWt.T, rdWt, "linear dWt")
+
+
+@pytest.mark.parametrize("M,K,N,p", [(4100, 1024, 384, 0.5), (4100, 1024, 384, 1.0), (4100, 1024, 384, 0.0), (8300, 1024, 1024, 0.3)])
+def test_linear_bwd_fused_launch(dev, M, K, N, p):
+    """Shapes whose dx and weight-gradient GEMMs both run on 128x128 tiles share one launch (dx tiles
+    behind the weight-gradient tiles): gradients against the oracle, exact zeros for an absent modality,
+    bit-identical on a second call."""
+    note(f"linear bwd fused launch M={M} K={K} N={N} p={p}")
+    assert _lib.tile_config(_lib.OP_BWD_DX, M, K, N)["block_m"] == 128 and _lib.tile_config(_lib.OP_BWD_DX, M, K, N)["block_n"] == 128
+    assert _lib.tile_config(_lib.OP_BWD_DW, M, K, N)["block_m"] == 128
+    gen = torch.Generator().manual_seed(M + N)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_linear("t", M, K, N, mask, seed=M, with_grad=True, w_std=0.05)
+    d = w.to(dev)
+    dx, dWv, dWt = masked_linear_backward(d.grad, d.x, d.Wv.T, d.Wt.T, d.mask)
+    rdx, rdWv, rdWt = cref.linear_bwd(w.grad, w.x, w.Wv, w.Wt, w.mask)
+    assert_close(dx, rdx, "dx")
+    assert_close(dWv.T, rdWv, "dWv")
+    assert_close(dWt.T, rdWt, "dWt")
+    if p == 1.0:
+        assert torch.count_nonzero(dWt) == 0
+    if p == 0.0:
+        assert torch.count_nonzero(dWv) == 0
+    again = masked_linear_backward(d.grad, d.x, d.Wv.T, d.Wt.T, d.mask)
+    for a, b in zip((dx, dWv, dWt), again):
+        assert torch.equal(a, b)
