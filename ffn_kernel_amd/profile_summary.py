@@ -66,9 +66,11 @@ def _roofline_kernels(workload: str):
     return _ours  # decode / linear workloads: every launch of one call
 
 
-def summarize(out: Path, workload: str, traffic_json: Path | None) -> str:
+def summarize(out: Path, workload: str, traffic_json: Path | None, min_pct: float = 0.5) -> str:
     lines = [f"workload: {workload}"]
     stats = _kernel_stats(out / "trace")
+    # counters are listed for the kernels that matter: at least min_pct of the traced kernel time
+    shown = {r["Name"] for r in stats if float(r["Percentage"]) >= min_pct} if stats else None
     if stats:
         lines += ["", "== rocprofv3 --kernel-trace --stats (ns) =="]
         for r in stats:
@@ -80,6 +82,8 @@ def summarize(out: Path, workload: str, traffic_json: Path | None) -> str:
     for sub in sorted(p.name for p in out.iterdir() if p.is_dir() and p.name not in ("trace", "cfetch", "cwrite")):
         for kernel, cs in sorted(_counters(out / sub).items()):
             if not _ours(kernel) and "Cijk" not in kernel:
+                continue
+            if shown is not None and kernel not in shown:
                 continue
             for c, v in sorted(cs.items()):
                 lines.append(f"{kernel[:100]:100s} {c:30s} n={len(v):3d} avg={sum(v) / len(v):.5g}")
@@ -118,8 +122,9 @@ def main() -> int:
     ap.add_argument("out", type=Path)
     ap.add_argument("--workload", required=True)
     ap.add_argument("--traffic-json", type=Path, default=None)
+    ap.add_argument("--min-pct", type=float, default=0.5, help="list counters of kernels with at least this share of the time")
     args = ap.parse_args()
-    sys.stdout.write(summarize(args.out, args.workload, args.traffic_json))
+    sys.stdout.write(summarize(args.out, args.workload, args.traffic_json, args.min_pct))
     return 0
 
 
