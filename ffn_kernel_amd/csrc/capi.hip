@@ -202,7 +202,12 @@ bool use_tile_path(int64_t M, int64_t d, int64_t h) {
 
 int down_splits(int64_t M, int64_t d, int64_t h) {
   if (use_dot_path(M, d, h)) return 1;
-  if (use_tile_path(M, d, h)) return stream_tile_down_splits((int)M, (int)d, (int)h);
+  if (use_tile_path(M, d, h)) {
+    // a forced factor (tuner) where every K range keeps the kernel's minimum of eight 128-element chunks
+    const int fs = forced_splits(), chunks = (int)(h / 128);
+    if (fs >= 1 && chunks - (int)cdiv64(chunks, fs) * (fs - 1) >= 8) return fs;
+    return stream_tile_down_splits((int)M, (int)d, (int)h);
+  }
   return stream_down_splits(d, h, stream_rows_per_block((int)M, false), stream_waves_per_block((int)M, false));
 }
 
