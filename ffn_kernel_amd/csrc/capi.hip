@@ -382,10 +382,10 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->block_k = 64;
   out->waves_m = gm.waves_m;
   out->waves_n = gm.waves_n;
-  out->lds_stages = 2;
   out->group_m = dual ? 8 : 4;
   out->split_k = splits;
   out->direct_lds = (contraction > 0 && contraction % 64 == 0) ? 1 : 0;
+  out->lds_stages = (tile == TILE_128x128_R4 && out->direct_lds) ? 4 : 2;
   if (op == FFNK_OP_FFN_DOWN && !stream) out->split_k = tiled_down_splits(M, K, N);
   if (op == FFNK_OP_LINEAR_FWD && linear_stream_kind(M, K, N)) {
     out->path = FFNK_PATH_STREAM;

@@ -16,6 +16,7 @@ hipError_t launch_splitk_gemm(int tile, const SplitKArgs& g, hipStream_t stream)
     case TILE_256x256_W4: return launch_grouped_splitk<Tiles::T1>(g, stream);
     case TILE_128x128_W4: return launch_grouped_splitk<Tiles::T2>(g, stream);
     case TILE_SMALL_W4: return launch_grouped_splitk<Tiles::T3>(g, stream);
+    case TILE_128x128_R4: return launch_grouped_splitk<Tiles::T4>(g, stream);
     default: return hipErrorInvalidValue;
   }
 }

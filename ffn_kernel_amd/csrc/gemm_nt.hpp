@@ -90,7 +90,7 @@ struct KMajorB {
 };
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool DUAL_, bool GATHER_A_, bool SCATTER_C_,
-          bool DIRECT_, int GROUP_M_, bool B_KMAJOR_ = false>
+          bool DIRECT_, int GROUP_M_, bool B_KMAJOR_ = false, int STAGES_ = 2>
 struct RoutedGemmCfg {
   static constexpr int BM = BM_;            // token rows per tile
   static constexpr int BN = BN_;            // B rows held in LDS per tile (DUAL: half gate, half up)
@@ -123,7 +123,13 @@ struct RoutedGemmCfg {
   static constexpr int TN = DUAL ? 2 * TN_OUT : TN_OUT;    // accumulator tiles per wave, N direction
   static constexpr int A_BYTES = BM * kRowBytes;           // slab layout
   static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  // More than two stages: a ring of K slabs with the loads STAGES - 1 slabs ahead (gemm_mainloop_ring) -
+  // for small tiles whose slab of MFMAs is shorter than the memory latency; one workgroup per CU.
+  static constexpr int STAGES = STAGES_;
+  static constexpr bool RING = STAGES_ > 2;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static_assert(STAGES_ >= 2 && STAGES_ <= 6 && STAGES_ * (BM_ + BN_) * kRowBytes <= 160 * 1024, "LDS stages");
+  static_assert(STAGES_ == 2 || (DIRECT_ && !B_KMAJOR_ && BM_ <= 128), "ring: direct path of the small tiles");
   static_assert(WTM % 32 == 0 && WTN_OUT % 32 == 0, "wave tile must be a multiple of 32x32");
   static_assert(NWAVES % 2 == 0, "lane mapping of the slab layout needs an even wave count");
   static_assert((BM / 16) % NWAVES == 0 && (BN / 16) % NWAVES == 0, "panel rows must split evenly over waves");
@@ -823,6 +829,156 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
 #endif
 }
 
+// s_waitcnt vmcnt(n) lgkmcnt(0) + s_barrier for a run-time n (the counter is an immediate).
+__device__ __forceinline__ void dma_wait_barrier_n(int n) {
+  switch (n) {
+#define FFNK_WB(N) case N: dma_wait_barrier<N>(); break;
+    FFNK_WB(0) FFNK_WB(1) FFNK_WB(2) FFNK_WB(3) FFNK_WB(4) FFNK_WB(5) FFNK_WB(6) FFNK_WB(7) FFNK_WB(8) FFNK_WB(9)
+    FFNK_WB(10) FFNK_WB(11) FFNK_WB(12) FFNK_WB(13) FFNK_WB(14) FFNK_WB(15) FFNK_WB(16) FFNK_WB(17) FFNK_WB(18)
+    FFNK_WB(19) FFNK_WB(20) FFNK_WB(21) FFNK_WB(22) FFNK_WB(23) FFNK_WB(24) FFNK_WB(25) FFNK_WB(26) FFNK_WB(27)
+    FFNK_WB(28) FFNK_WB(29) FFNK_WB(30) FFNK_WB(31) FFNK_WB(32) FFNK_WB(33) FFNK_WB(34) FFNK_WB(35) FFNK_WB(36)
+#undef FFNK_WB
+    default: dma_wait_barrier<0>(); break;
+  }
+}
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// =============================================================================================
+// Ring of S > 2 stages for the small tiles (32x32x16 MFMAs).  A 128x128 tile's slab is 512 cycles of
+// MFMAs per wave, less than the latency of the loads that feed the next one: behind two stages the K loop
+// runs at the memory latency (0.8 us per slab measured against 0.3 us of MFMAs).  Here slab kt + S - 1 is
+// loaded while slab kt is computed: its first quarter of loads goes out behind the last K step of slab
+// kt - 1 (right after the barrier that frees its stage), the other three quarters behind the first three
+// K steps of slab kt - at most one load per MFMA, which is what the address unit takes.  One barrier per
+// slab, before its last K step: every wave has read the last fragments of the stage before, and slab
+// kt + 1 has landed (loads complete in order, so "at most (S - 2) slabs of loads outstanding").  Same
+// source-order schedule as the 256-row tiles.
+// =============================================================================================
+template <class Cfg>
+__device__ __forceinline__ void gemm_mainloop_ring(const TileLanes<Cfg>& tl,
+                                                   const uint16_t* const (&baseA)[TileLanes<Cfg>::NJA],
+                                                   const uint32_t (&offA)[TileLanes<Cfg>::NJA],
+                                                   const uint16_t* const (&baseB)[TileLanes<Cfg>::NJB],
+                                                   const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
+                                                   uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN]) {
+  static_assert(Cfg::RING && !Cfg::MFMA16, "ring schedule of the small direct tiles");
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN, S = Cfg::STAGES, D = S - 1;
+  constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
+  constexpr int L = NJA + NJB;
+  constexpr int STAGE = Cfg::STAGE_BYTES, A_BYTES = Cfg::A_BYTES;
+  constexpr int NM = TM * TN, ND = TM + TN;
+  constexpr int LQ = (L + 3) / 4;            // loads per K step (a slab's loads go out over four steps)
+  constexpr int RPM = (ND + NM - 1) / NM;    // fragment reads behind each MFMA
+  constexpr int LPM = (LQ + NM - 1) / NM;    // loads behind each MFMA
+  static_assert((S - 1) * L + LQ <= 36, "dma_wait_barrier_n covers this many loads");
+  const int wave = tl.wave_s;
+
+  auto wave_uniform = [](const uint16_t* p) {
+    if (!Cfg::DUAL) return reinterpret_cast<void*>(const_cast<uint16_t*>(p));
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+  };
+  __amdgpu_buffer_rsrc_t rsA[NJA], rsB[NJB];
+#pragma unroll
+  for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseA[j]), 0, 0xffffffff, 0x00020000);
+#pragma unroll
+  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
+  uint32_t koff[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) koff[s] = lds_swizzle(tl.lr, 2 * s + tl.lh);
+  const uint32_t a_base = (uint32_t)(tl.wm * Cfg::WTM) * kRowBytes;
+  uint32_t b_base[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) b_base[tn] = A_BYTES + (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
+
+  zero_acc<Cfg>(acc);
+  const int nk = k_len / kBK;
+
+  bf16x8_t fa[2][TM], fb[2][TN];
+  auto read_frag = [&](int buf, int stage, int ks, int r) {
+    const uint8_t* st = lds + stage * STAGE;
+    if (r < TN) fb[buf][r] = *reinterpret_cast<const bf16x8_t*>(st + b_base[r] + koff[ks]);
+    else fa[buf][r - TN] = *reinterpret_cast<const bf16x8_t*>(st + a_base + (r - TN) * 32 * kRowBytes + koff[ks]);
+  };
+  auto load = [&](int l, int stage, int kt) {
+    uint8_t* st = lds + stage * STAGE;
+    const int ko = kt * kRowBytes;
+    if (l < NJB)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l - NJB], FFNK_LDS_PTR(st + ((l - NJB) * NWAVES + wave) * 1024), 16,
+                                               offA[l - NJB], ko, 0, 0);
+  };
+  // One K step: the MFMAs on fragment buffer `cur`; behind them the fragment reads of (stage_next, ks_next)
+  // into the other buffer and loads [l0, l0 + LQ) of slab kt_dma into stage_dma.
+  auto step = [&](int cur, int stage_next, int ks_next, bool reads, bool dma, int l0, int stage_dma, int kt_dma) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < NM; ++q) {
+      acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][q % TN], fa[cur][q / TN], acc[q / TN][q % TN], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = q * RPM; r < (q + 1) * RPM && r < ND; ++r)
+        if (reads) read_frag(cur ^ 1, stage_next, ks_next, r);
+#pragma unroll
+      for (int i = q * LPM; i < (q + 1) * LPM && i < LQ; ++i)
+        if (dma && l0 + i < L) load(l0 + i, stage_dma, kt_dma);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // Slab kt in stage U.  On entry slabs up to kt + D - 1 are issued, and the first quarter of slab kt + D.
+  auto body = [&](auto stage_tag, int kt, bool steady) {
+    constexpr int U = decltype(stage_tag)::value, UN = (U + 1) % S, UP = (U + S - 1) % S;
+    const bool far = steady || kt + D < nk;        // slab kt + D exists
+    step(0, U, 1, true, far, LQ, UP, kt + D);
+    step(1, U, 2, true, far, 2 * LQ, UP, kt + D);
+    step(0, U, 3, true, far, 3 * LQ, UP, kt + D);
+    if (steady) {
+      dma_wait_barrier<(S - 2) * L>();
+    } else {
+      const int last = kt + D < nk ? kt + D : nk - 1;  // last slab issued so far
+      dma_wait_barrier_n(last > kt + 1 ? (last - kt - 1) * L : 0);
+    }
+    step(1, UN, 0, steady || kt + 1 < nk, steady || kt + S < nk, 0, U, kt + S);
+  };
+
+  // Head of the tile: slabs 0 .. D - 1 whole and the first quarter of slab D, as the steady schedule leaves them.
+  int issued = 0;
+#pragma unroll
+  for (int j = 0; j < D; ++j)
+    if (j < nk) {
+#pragma unroll
+      for (int l = 0; l < L; ++l) load(l, j, j);
+      issued += L;
+    }
+  if (D < nk) {
+#pragma unroll
+    for (int l = 0; l < LQ && l < L; ++l) load(l, D % S, D);
+    issued += LQ < L ? LQ : L;
+  }
+  dma_wait_barrier_n(issued - L);  // slab 0 has landed
+#pragma unroll
+  for (int r = 0; r < ND; ++r) read_frag(0, 0, 0, r);
+
+  int kt = 0;
+  for (; kt + 2 * S - 1 < nk; kt += S) static_for<0, S>([&](auto u) { body(u, kt + decltype(u)::value, true); });
+  for (; kt < nk; kt += S)
+    static_for<0, S>([&](auto u) {
+      if (kt + decltype(u)::value < nk) body(u, kt + decltype(u)::value, false);
+    });
+#endif
+}
+
 // Main loop of a direct-path tile, by the tile's MFMA shape.
 template <class Cfg>
 __device__ __forceinline__ void gemm_mainloop_direct(const TileLanes<Cfg>& tl,
@@ -833,6 +989,7 @@ __device__ __forceinline__ void gemm_mainloop_direct(const TileLanes<Cfg>& tl,
                                                      uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN],
                                                      const KMajorB& kb = KMajorB()) {
   if constexpr (Cfg::MFMA16) gemm_mainloop_fixed16<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc);
+  else if constexpr (Cfg::RING) gemm_mainloop_ring<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc);
   else gemm_mainloop_slab_dma<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
 }
 

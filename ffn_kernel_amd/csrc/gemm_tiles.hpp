@@ -15,6 +15,8 @@ struct PlainTiles {
   using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
   using T2 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
   using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
+  // 128x128 behind a ring of four LDS stages (direct path; otherwise the two-stage tile)
+  using T4 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain, false, DIRECT ? 4 : 2>;
 };
 
 // The same tiles over K-major weights ([K, N] rows, N contiguous; direct path only).
@@ -24,6 +26,7 @@ struct KMajorTiles {
   using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
   using T2 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
   using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
+  using T4 = T2;  // no ring over K-major weights
 };
 
 // SwiGLU tiles: BN = gate rows + up rows held in LDS, i.e. BN / 2 output columns.
@@ -33,6 +36,7 @@ struct DualTiles {
   using T1 = RoutedGemmCfg<256, 256, 2, 2, true, true, false, DIRECT, kGroupM>;
   using T2 = RoutedGemmCfg<128, 128, 2, 2, true, true, false, DIRECT, kGroupM>;
   using T3 = RoutedGemmCfg<64, 128, 2, 2, true, true, false, DIRECT, kGroupM>;
+  using T4 = RoutedGemmCfg<128, 128, 2, 2, true, true, false, DIRECT, kGroupM, false, DIRECT ? 4 : 2>;
 };
 
 template <class Tiles>
@@ -42,6 +46,7 @@ inline hipError_t dispatch_tile(int tile, const GemmArgs& g, hipStream_t stream)
     case TILE_256x256_W4: return launch_routed_gemm<typename Tiles::T1>(g, stream);
     case TILE_128x128_W4: return launch_routed_gemm<typename Tiles::T2>(g, stream);
     case TILE_SMALL_W4: return launch_routed_gemm<typename Tiles::T3>(g, stream);
+    case TILE_128x128_R4: return launch_routed_gemm<typename Tiles::T4>(g, stream);
     default: return hipErrorInvalidValue;
   }
 }

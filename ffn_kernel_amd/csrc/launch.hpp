@@ -15,7 +15,8 @@ enum TileId : int {
   TILE_256x256_W4 = 1,  // 256x256 macro tile, 4 waves (2x2), wave tile 128x128
   TILE_128x128_W4 = 2,  // 128x128 macro tile, 4 waves (2x2), wave tile 64x64
   TILE_SMALL_W4 = 3,    // 128x64 (plain) or 64x128 holding 64 gate + 64 up rows (SwiGLU), 4 waves
-  TILE_COUNT = 4
+  TILE_128x128_R4 = 4,  // 128x128, 4 waves, ring of four LDS stages (one workgroup per CU; long contractions, few tiles)
+  TILE_COUNT = 5
 };
 
 // The two 256x256 tiles: past one round of the chip they run whole rounds first and the remainder apart.

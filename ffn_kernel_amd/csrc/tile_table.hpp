@@ -88,7 +88,7 @@ inline double routed_plan_cost(int64_t M, int64_t n_out, int64_t K, int tile, in
   const TileGeom t = tile_geom(tile, false);
   const int64_t tiles = (cdiv64(M, t.block_m) + 1) * cdiv64(n_out, t.block_n_out);
   const int64_t slots = (int64_t)kCus * (tile == TILE_SMALL_W4 ? 3 : tile == TILE_128x128_W4 ? 2 : 1);
-  const double t_slab = (tile == TILE_256x256_W8 || tile == TILE_256x256_W4) ? 1.2 : 0.8;
+  const double t_slab = (tile == TILE_256x256_W8 || tile == TILE_256x256_W4) ? 1.2 : tile == TILE_128x128_R4 ? 0.4 : 0.8;
   const int64_t slabs = cdiv64(cdiv64(K, 64), splits);
   const double reduce = splits > 1 ? (double)splits * (double)M * (double)n_out * 8.0 / 4.0e6 : 0.0;
   if (tile == TILE_256x256_W8 && splits == 1 && K % 64 == 0 && tiles > slots) {

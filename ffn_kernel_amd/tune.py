@@ -9,9 +9,14 @@ The lattice is (tile id) x (split-K factor) per operation, layer shape and M buc
   * MaskedLinear forward: (tile, split-K factor) of the routed GEMM, whole call;
   * MaskedLinear backward: the weight-gradient GEMM's split-K factor, whole call.
 Every candidate is forced through ffnk_debug_force_tile / ffnk_debug_force_splits and timed min-of-k;
-the baseline is the library's rules and cost model alone (ffnk_debug_force_tile(-2)).  Wherever the best
-candidate beats the baseline by more than --margin, an entry goes into csrc/tile_table_gen.hpp, which
-pick_routed_plan / pick_routed_tile / pick_splitk_tile (csrc/tile_table.hpp) consult before the rules.
+the baseline is the library's rules and cost model alone (ffnk_debug_force_tile(-2)).  The host never
+knows how many rows each group holds, and a tile's time jumps where a group's tile count crosses a
+multiple of the CU count, so one mask says little about a bucket: every bucket is measured on several
+scenarios (its upper end with an i.i.d. mask, its upper end with contiguous spans, a point inside it).
+All candidates run the first scenario; the few that beat the baseline there run the others.  An entry
+goes into csrc/tile_table_gen.hpp, which pick_routed_plan / pick_routed_tile / pick_splitk_tile
+(csrc/tile_table.hpp) consult before the rules, only for a candidate that loses on no scenario and whose
+geometric-mean time beats the baseline by more than --margin.
 
     python -m ffn_kernel_amd.tune                 # sweep, print the comparison
     python -m ffn_kernel_amd.tune --emit          # ... and rewrite csrc/tile_table_gen.hpp (then rebuild)
@@ -30,7 +35,7 @@ import torch
 from . import _lib
 from .ops import masked_linear_backward, masked_linear_forward
 
-TILES = {0: "256x256/8w", 1: "256x256/4w", 2: "128x128/4w", 3: "small/4w"}
+TILES = {0: "256x256/8w", 1: "256x256/4w", 2: "128x128/4w", 3: "small/4w", 4: "128x128/ring4"}
 SPLITS = (1, 2, 3, 4, 6, 7, 8, 12, 14, 16)
 TUNED_PLAIN, TUNED_DUAL, TUNED_SPLITK = 0, 1, 2
 GEN_PATH = Path(__file__).resolve().parent / "csrc" / "tile_table_gen.hpp"
@@ -134,97 +139,180 @@ def _valid_splits(contraction, M):
     return out
 
 
-def tune_ffn(d, h, bucket, trials, dev, ev):
-    lo, M = bucket
-    gen = torch.Generator(device=dev).manual_seed(M)
-    x = _randn((M, d), 1.0, gen, dev)
-    mask = torch.rand(M, generator=gen, device=dev) < 0.5
+def _span_mask(M, frac, n_seq, gen, dev):
+    """n_seq sequences of M / n_seq rows, each with one contiguous span of about frac of its rows set."""
+    mask = torch.zeros(M, dtype=torch.bool, device=dev)
+    seq = max(1, M // n_seq)
+    span = max(1, int(seq * frac))
+    for b in range(n_seq):
+        start = b * seq + int(torch.randint(0, max(1, seq - span), (1,), generator=gen, device=dev))
+        mask[start:start + span] = True
+    return mask
+
+
+def _scenarios(bucket, gen, dev):
+    """[(M, mask)]: the bucket's upper end with an i.i.d. mask, the same with spans, and a point inside."""
+    lo, hi = bucket
+    mid = lo + (hi - lo) * 2 // 5
+    return [(hi, torch.rand(hi, generator=gen, device=dev) < 0.5),
+            (hi, _span_mask(hi, 0.3, 4, gen, dev)),
+            (mid, _span_mask(mid, 0.6, 2, gen, dev))]
+
+
+def _shortlist(base0, cand0, margin, keep=3):
+    """Keys of the candidates that beat the baseline on the first scenario, best first, at most `keep`."""
+    good = sorted((t, k) for k, t in cand0.items() if t < base0 * (1 - margin))
+    return [k for _, k in good[:keep]]
+
+
+def _geomean(xs):
+    p = 1.0
+    for x in xs:
+        p *= x
+    return p ** (1.0 / len(xs))
+
+
+def _select(base, cand, margin):
+    """(key, geometric-mean ratio) of the best candidate measured on every scenario that loses on none and
+    beats the baseline's geometric mean by more than margin; (None, 1.0) when there is none."""
+    best, best_r = None, 1.0 - margin
+    for k, ts in cand.items():
+        if len(ts) != len(base) or any(t > b * 1.01 for t, b in zip(ts, base)):
+            continue
+        r = _geomean([t / b for t, b in zip(ts, base)])
+        if r < best_r:
+            best, best_r = k, r
+    return best, (best_r if best is not None else 1.0)
+
+
+def tune_ffn(d, h, bucket, trials, dev, ev, margin):
+    lo, hi = bucket
+    gen = torch.Generator(device=dev).manual_seed(hi)
     W = {k: _randn((h, d), 0.02, gen, dev) for k in ("w1", "w3", "u1", "u3")}
     W.update({k: _randn((d, h), 0.02, gen, dev) for k in ("w2", "u2")})
+    scen = [(_randn((M, d), 1.0, gen, dev), mask) for M, mask in _scenarios(bucket, gen, dev)]
+    base_up, base_down = [], []
     with _Forced(-2, -1):
-        base_up, base_down = _ffn_stage_ms(x, W, mask, trials, ev)
-        base_cfg = {"up": _lib.tile_config(_lib.OP_FFN_UP, M, d, h), "down": _lib.tile_config(_lib.OP_FFN_DOWN, M, d, h)}
-    ups, downs = {}, {}
+        for x, mask in scen:
+            u, dn = _ffn_stage_ms(x, W, mask, trials, ev)
+            base_up.append(u)
+            base_down.append(dn)
+        base_cfg = {"up": _lib.tile_config(_lib.OP_FFN_UP, hi, d, h), "down": _lib.tile_config(_lib.OP_FFN_DOWN, hi, d, h)}
+
+    def run(tile, s, x, mask):
+        """(up ms, down ms) under the override, or None when the shape does not take the factor."""
+        with _Forced(tile, s):
+            if _lib.tile_config(_lib.OP_FFN_DOWN, x.shape[0], d, h)["split_k"] != s:
+                return None
+            return _ffn_stage_ms(x, W, mask, trials, ev)
+
+    ups0, downs0 = {}, {}
     for tile in TILES:
-        for s in _valid_splits(h, M):
+        for s in _valid_splits(h, hi):
             if tile == 1 and s > 1:
                 continue  # the four-wave 256x256 tile is not run split
-            with _Forced(tile, s):
-                got_s = _lib.tile_config(_lib.OP_FFN_DOWN, M, d, h)["split_k"]
-                if got_s != s:
-                    continue  # the shape does not take this factor
-                u, dn = _ffn_stage_ms(x, W, mask, trials, ev)
-            ups[tile] = min(ups.get(tile, float("inf")), u)
-            downs[(tile, s)] = dn
-    return {"op": "ffn_fwd", "d": d, "h": h, "m_lo": lo, "m_hi": M, "rules": base_cfg, "rules_up_ms": base_up,
-            "rules_down_ms": base_down, "up_ms": ups, "down_ms": downs}
+            got = run(tile, s, *scen[0])
+            if got is None:
+                continue
+            if s == 1:
+                ups0[tile] = got[0]
+            downs0[(tile, s)] = got[1]
+    ups = {t: [ups0[t]] for t in _shortlist(base_up[0], ups0, margin)}
+    downs = {k: [downs0[k]] for k in _shortlist(base_down[0], downs0, margin)}
+    for key in sorted(set((t, 1) for t in ups) | set(downs)):
+        for x, mask in scen[1:]:
+            got = run(key[0], key[1], x, mask)
+            if got is None:
+                break
+            if key[1] == 1 and key[0] in ups:
+                ups[key[0]].append(got[0])
+            if key in downs:
+                downs[key].append(got[1])
+    return {"op": "ffn_fwd", "d": d, "h": h, "m_lo": lo, "m_hi": hi, "rules": base_cfg, "rules_up_ms": base_up,
+            "rules_down_ms": base_down, "up_first_ms": ups0, "down_first_ms": downs0, "up_ms": ups, "down_ms": downs}
 
 
-def tune_linear_fwd(K, N, bucket, trials, dev):
-    lo, M = bucket
-    gen = torch.Generator(device=dev).manual_seed(M + 1)
-    x = _randn((M, K), 1.0, gen, dev)
-    mask = torch.rand(M, generator=gen, device=dev) < 0.5
-    Wv, Wt = _randn((N, K), 0.02, gen, dev), _randn((N, K), 0.02, gen, dev)
-    fn = lambda: masked_linear_forward(x, Wv.T, Wt.T, mask)
+def _tune_call(make_fn, scen_inputs, candidates, trials, margin):
+    """Whole-call counterpart of tune_ffn's search: make_fn(inputs) -> callable; candidates yields
+    (key, tile, splits, accept(M) -> bool).  Returns (baseline ms per scenario, {key: ms on the first
+    scenario}, {key: [ms per scenario]} for the shortlist)."""
+    fns = [make_fn(inp) for inp in scen_inputs]
     with _Forced(-2, -1):
-        base = _call_ms(fn, trials)
-        base_cfg = _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, N)
-    cand = {}
+        base = [_call_ms(fn, trials) for fn in fns]
+    first = {}
+    for key, tile, s, accept in candidates:
+        with _Forced(tile, s):
+            if accept(scen_inputs[0][0].shape[0]):
+                first[key] = (_call_ms(fns[0], trials), tile, s, accept)
+    first_ms = {k: v[0] for k, v in first.items()}
+    full = {}
+    for key in _shortlist(base[0], first_ms, margin):
+        _, tile, s, accept = first[key]
+        ts = [first_ms[key]]
+        with _Forced(tile, s):
+            for inp, fn in zip(scen_inputs[1:], fns[1:]):
+                if not accept(inp[0].shape[0]):
+                    break
+                ts.append(_call_ms(fn, trials))
+        full[key] = ts
+    return base, first_ms, full
+
+
+def tune_linear_fwd(K, N, bucket, trials, dev, margin):
+    lo, hi = bucket
+    gen = torch.Generator(device=dev).manual_seed(hi + 1)
+    Wv, Wt = _randn((N, K), 0.02, gen, dev), _randn((N, K), 0.02, gen, dev)
+    scen = [(_randn((M, K), 1.0, gen, dev), mask) for M, mask in _scenarios(bucket, gen, dev)]
+    with _Forced(-2, -1):
+        base_cfg = _lib.tile_config(_lib.OP_LINEAR_FWD, hi, K, N)
+    cands = []
     if base_cfg["path"] == _lib.PATH_MFMA_TILED:
         for tile in TILES:
-            for s in _valid_splits(K, M):
+            for s in _valid_splits(K, hi):
                 if tile == 1 and s > 1:
                     continue
-                with _Forced(tile, s):
-                    if _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, N)["split_k"] != s:
-                        continue
-                    cand[(tile, s)] = _call_ms(fn, trials)
-    return {"op": "linear_fwd", "K": K, "N": N, "m_lo": lo, "m_hi": M, "rules": base_cfg, "rules_ms": base, "ms": cand}
+                cands.append(((tile, s), tile, s,
+                              lambda M, s=s: _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, N)["split_k"] == s))
+    base, first, full = _tune_call(lambda inp: (lambda: masked_linear_forward(inp[0], Wv.T, Wt.T, inp[1])),
+                                   scen, cands, trials, margin)
+    return {"op": "linear_fwd", "K": K, "N": N, "m_lo": lo, "m_hi": hi, "rules": base_cfg, "rules_ms": base,
+            "first_ms": first, "ms": full}
 
 
-def tune_linear_bwd(K, N, bucket, trials, dev):
-    lo, M = bucket
-    gen = torch.Generator(device=dev).manual_seed(M + 2)
-    x = _randn((M, K), 1.0, gen, dev)
-    g = _randn((M, N), 1.0, gen, dev)
-    mask = torch.rand(M, generator=gen, device=dev) < 0.5
+def tune_linear_bwd(K, N, bucket, trials, dev, margin):
+    lo, hi = bucket
+    gen = torch.Generator(device=dev).manual_seed(hi + 2)
     Wv, Wt = _randn((N, K), 0.02, gen, dev), _randn((N, K), 0.02, gen, dev)
-    fn = lambda: masked_linear_backward(g, x, Wv.T, Wt.T, mask)
+    scen = [(_randn((M, K), 1.0, gen, dev), mask, _randn((M, N), 1.0, gen, dev)) for M, mask in _scenarios(bucket, gen, dev)]
     with _Forced(-2, -1):
-        base = _call_ms(fn, trials)
-        base_cfg = _lib.tile_config(_lib.OP_BWD_DW, M, K, N)
-    cand = {}
-    slabs = max(1, (M // 2) // 64)
-    for s in SPLITS:
-        if s > slabs:
-            continue
-        with _Forced(-2, s):
-            cand[s] = _call_ms(fn, trials)
-    return {"op": "linear_bwd", "K": K, "N": N, "m_lo": lo, "m_hi": M, "rules": base_cfg, "rules_ms": base, "ms": cand}
+        base_cfg = _lib.tile_config(_lib.OP_BWD_DW, hi, K, N)
+    slabs = max(1, (lo // 4) // 64)  # every factor must leave whole slabs in the smaller group of the smallest scenario
+    cands = [(s, -2, s, lambda M: True) for s in SPLITS if s <= slabs]
+    base, first, full = _tune_call(lambda inp: (lambda: masked_linear_backward(inp[2], inp[0], Wv.T, Wt.T, inp[1])),
+                                   scen, cands, trials, margin)
+    return {"op": "linear_bwd", "K": K, "N": N, "m_lo": lo, "m_hi": hi, "rules": base_cfg, "rules_ms": base,
+            "first_ms": first, "ms": full}
 
 
 def plans_from(records, margin):
-    """Table entries (op, m_lo, m_hi, k, n, tile, splits) for every record whose best candidate beats the
-    rules by more than `margin`."""
+    """Table entries (op, m_lo, m_hi, k, n, tile, splits) for every record with a candidate that loses on
+    no scenario and beats the rules' geometric-mean time by more than `margin`."""
     out = []
     for r in records:
         if r["op"] == "ffn_fwd":
-            if r["up_ms"]:
-                tile = min(r["up_ms"], key=r["up_ms"].get)
-                if r["up_ms"][tile] < r["rules_up_ms"] * (1 - margin):
-                    out.append((TUNED_DUAL, r["m_lo"], r["m_hi"], r["d"], r["h"], tile, 1))
-            if r["down_ms"]:
-                tile, s = min(r["down_ms"], key=r["down_ms"].get)
-                if r["down_ms"][(tile, s)] < r["rules_down_ms"] * (1 - margin):
-                    out.append((TUNED_PLAIN, r["m_lo"], r["m_hi"], r["h"], r["d"], tile, s))
-        elif r["op"] == "linear_fwd" and r["ms"]:
-            tile, s = min(r["ms"], key=r["ms"].get)
-            if r["ms"][(tile, s)] < r["rules_ms"] * (1 - margin):
-                out.append((TUNED_PLAIN, r["m_lo"], r["m_hi"], r["K"], r["N"], tile, s))
-        elif r["op"] == "linear_bwd" and r["ms"]:
-            s = min(r["ms"], key=r["ms"].get)
-            if r["ms"][s] < r["rules_ms"] * (1 - margin):
+            tile, _ = _select(r["rules_up_ms"], r["up_ms"], margin)
+            if tile is not None:
+                out.append((TUNED_DUAL, r["m_lo"], r["m_hi"], r["d"], r["h"], tile, 1))
+            key, _ = _select(r["rules_down_ms"], r["down_ms"], margin)
+            if key is not None:
+                out.append((TUNED_PLAIN, r["m_lo"], r["m_hi"], r["h"], r["d"], key[0], key[1]))
+        elif r["op"] == "linear_fwd":
+            key, _ = _select(r["rules_ms"], r["ms"], margin)
+            if key is not None:
+                out.append((TUNED_PLAIN, r["m_lo"], r["m_hi"], r["K"], r["N"], key[0], key[1]))
+        elif r["op"] == "linear_bwd":
+            s, _ = _select(r["rules_ms"], r["ms"], margin)
+            if s is not None:
                 tile = {(256, 256): 0, (128, 128): 2}.get((r["rules"]["block_m"], r["rules"]["block_n"]), 2)
                 out.append((TUNED_SPLITK, r["m_lo"], r["m_hi"], r["N"], r["K"], tile, s))  # R = N, Cc = K (dW stored [N, K])
     # one entry per key: a linear layer and an FFN's down projection can share (k, n); keep the first
@@ -246,8 +334,8 @@ def render_header(plans) -> str:
     return "\n".join(lines)
 
 
-def _fmt(d):
-    return "  ".join(f"{k}={v:.3f}" for k, v in d.items())
+def _fmt_list(ts):
+    return "/".join(f"{t:.3f}" for t in ts)
 
 
 def main(argv=None) -> int:
@@ -267,30 +355,33 @@ def main(argv=None) -> int:
     ev = _Events()
     buckets = [BUCKETS[1], BUCKETS[4]] if args.quick else BUCKETS
     records = []
+
+    def ratios(base, cand):
+        return "  ".join(f"{k}:" + "/".join(f"{t / b_:.2f}" for t, b_ in zip(ts, base)) for k, ts in cand.items()) or "-"
+
     for d, h in FFN_LAYERS:
         for b in buckets:
             if b[1] * h * 2 > 4 << 30:
                 continue
-            r = tune_ffn(d, h, b, args.trials, dev, ev)
+            r = tune_ffn(d, h, b, args.trials, dev, ev, args.margin)
             records.append(r)
-            print(f"ffn_fwd    d={d:5d} h={h:5d} M<={b[1]:6d} | rules up {r['rules_up_ms']:.3f} "
-                  f"(tile {r['rules']['up']['block_m']}x{r['rules']['up']['block_n']}/{r['rules']['up']['waves_m'] * r['rules']['up']['waves_n']}w)"
-                  f" down {r['rules_down_ms']:.3f} | up by tile: {_fmt({TILES[k]: v for k, v in r['up_ms'].items()})}"
-                  f" | best down: {min(r['down_ms'], key=r['down_ms'].get)} {min(r['down_ms'].values()):.3f}", flush=True)
+            up = r["rules"]["up"]
+            print(f"ffn_fwd    d={d:5d} h={h:5d} M<={b[1]:6d} | rules up {_fmt_list(r['rules_up_ms'])} "
+                  f"(tile {up['block_m']}x{up['block_n']}/{up['waves_m'] * up['waves_n']}w) down {_fmt_list(r['rules_down_ms'])}"
+                  f" | up tile:ratio per scenario {ratios(r['rules_up_ms'], r['up_ms'])}"
+                  f" | down (tile, splits):ratio {ratios(r['rules_down_ms'], r['down_ms'])}", flush=True)
     for K, N in LINEAR_LAYERS:
         for b in buckets:
-            r = tune_linear_fwd(K, N, b, args.trials, dev)
+            r = tune_linear_fwd(K, N, b, args.trials, dev, args.margin)
             records.append(r)
-            best = min(r["ms"], key=r["ms"].get) if r["ms"] else None
-            print(f"linear_fwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {r['rules_ms']:.3f} | best {best} "
-                  f"{r['ms'][best] if best else float('nan'):.3f}", flush=True)
-            r = tune_linear_bwd(K, N, b, args.trials, dev)
+            print(f"linear_fwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} | (tile, splits):ratio "
+                  f"{ratios(r['rules_ms'], r['ms'])}", flush=True)
+            r = tune_linear_bwd(K, N, b, args.trials, dev, args.margin)
             records.append(r)
-            best = min(r["ms"], key=r["ms"].get)
-            print(f"linear_bwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {r['rules_ms']:.3f} (splits {r['rules']['split_k']}) | "
-                  f"by splits: {_fmt({str(k): v for k, v in r['ms'].items()})}", flush=True)
+            print(f"linear_bwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} (splits {r['rules']['split_k']}) | "
+                  f"splits:ratio {ratios(r['rules_ms'], r['ms'])}", flush=True)
     plans = plans_from(records, args.margin)
-    print(f"{len(plans)} measured plans beat the rules by more than {args.margin:.0%}:")
+    print(f"{len(plans)} measured plans lose on no scenario and beat the rules by more than {args.margin:.0%}:")
     for e in plans:
         print("   op=%d M in [%d, %d] k=%d n=%d -> tile %d, splits %d" % e)
     if args.json:

@@ -199,7 +199,7 @@ def test_measured_plans_are_consulted_before_the_rules():
     text = tune.GEN_PATH.read_text()
     entries = [tuple(map(int, e)) for e in re.findall(r"^\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},$", text, re.M)]
     assert tune.render_header(entries) == text
-    geom = {0: (256, 256, 8), 1: (256, 256, 4), 2: (128, 128, 4)}
+    geom = {0: (256, 256, 8), 1: (256, 256, 4), 2: (128, 128, 4), 4: (128, 128, 4)}
     lib = _lib.load()
     checked = 0
     for op, lo, hi, k, n, tile, splits in entries:

@@ -765,11 +765,11 @@ def force_tile():
         lib.ffnk_debug_force_tile(-1)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("M,K,N,p", [(700, 256, 512, 0.5), (333, 192, 320, 0.3), (1100, 1024, 264, 1.0)])
 def test_forced_tile_linear_fwd_bwd(dev, force_tile, tile, M, K, N, p):
     """Each of the four tile shapes every GEMM family is compiled for (256x256 with 8 or 4 waves,
-    128x128, 128x64) runs the MaskedLinear forward and backward: the table alone never picks all of
+    128x128, 128x64, 128x128 behind a four-stage ring) runs the MaskedLinear forward and backward: the table alone never picks all of
     them at test sizes."""
     note(f"forced tile {tile}: linear fwd+bwd M={M} K={K} N={N} p={p}")
     gen = torch.Generator().manual_seed(M + tile)
@@ -790,7 +790,7 @@ def test_forced_tile_linear_fwd_bwd(dev, force_tile, tile, M, K, N, p):
         assert torch.count_nonzero(dWt) == 0
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("M,d,h,p", [(700, 256, 512, 0.5), (300, 128, 320, 0.4)])
 def test_forced_tile_ffn_fwd_bwd(dev, force_tile, tile, M, d, h, p):
     note(f"forced tile {tile}: ffn fwd+bwd M={M} d={d} h={h}")
