@@ -167,7 +167,7 @@ def _decode_rooflines(dev, weight_sets, steps: int) -> list:
         x, mask = wl.cfg5_inputs(M, kind)
         x, mask = x.to(dev), mask.to(dev)
         calls = [wl.FFNWorkload("d", x, W, mask).op_args() for W in weight_sets]
-        for i in range(6):
+        for i in range(20):
             MaskedFFN.apply(*calls[i % ns])
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -245,8 +245,10 @@ def _bench_linear(args, dev) -> dict:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default: 20 for cfg4, 200 for the microsecond-scale workloads, whose "
+                         "first launches after a synchronisation would otherwise dominate)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps first (default: 5, or 20 with 200 steps)")
     ap.add_argument("--workload", default="cfg4")
     ap.add_argument("--cpu-rows", type=int, default=1 << 30,
                     help="upper bound on the rows of the workload timed on the CPU (0 = skip); the sample is "
@@ -254,6 +256,11 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true",
                     help="cfg4 only: skip the decode-shape measurements (roofline_decode), e.g. under a profiler")
     args = ap.parse_args()
+    big = args.workload in ("cfg4", "gemm_ref", "copy1g")
+    if args.steps is None:
+        args.steps = 20 if big else 200
+    if args.warmup is None:
+        args.warmup = 5 if big else 20
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (rows are independent, so more GPUs "
               "would each run this same kernel on their slice of M)", file=sys.stderr)
@@ -396,7 +403,7 @@ def main() -> int:
     }
     if args.workload == "cfg4" and not args.no_decode:
         # The same layer at decode sizes (HBM-bound): the cfg4 weights plus two more sets rotate.
-        result["roofline_decode"] = _decode_rooflines(dev, more_weight_sets(w.W), steps=max(args.steps, 30))
+        result["roofline_decode"] = _decode_rooflines(dev, more_weight_sets(w.W), steps=max(args.steps, 200))
     if args.cpu_rows > 0:
         result["cpu_baseline"] = _cpu_baseline_ffn(w_cpu, min(args.cpu_rows, M))
     print(json.dumps(result), flush=True)
