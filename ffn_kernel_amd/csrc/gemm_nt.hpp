@@ -674,7 +674,7 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
 //  * A slab is two K steps of 32.  A step runs its TM x TN MFMAs row group by row group: the token
 //    fragment of a group (16 rows x 32 K) is single-buffered and re-read in place for the next step as
 //    soon as the group's last MFMA has issued (a whole step ahead of its next use); the TN weight
-//    fragments are double-buffered and read behind the first MFMAs of the previous step.
+//    fragments are double-buffered and read during the previous step, one behind the middle MFMA of each row group.
 //  * One barrier per slab, behind the first two row groups of the slab's second step: by then every
 //    fragment read of the stage has returned (the last one was issued two groups earlier) and the next
 //    slab, whose last loads went out more than half a slab before, has landed.
@@ -700,7 +700,7 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   constexpr int BAR = 2 * TN;            // MFMAs of a slab's second step ahead of the barrier (two row groups)
   constexpr int LEV = 4;                 // one load behind every fourth MFMA
   constexpr int L1 = (NM - BAR) / LEV;   // loads of the slab after next that go out in the second step
-  static_assert(TM >= 3 && L1 >= 1 && L1 <= L && (L - L1) * LEV <= NM, "schedule does not fit this wave tile");
+  static_assert(TM >= 3 && TM >= TN && L1 >= 1 && L1 <= L && (L - L1) * LEV <= NM, "schedule does not fit this wave tile");
   const int wave = tl.wave_s;
 
   auto wave_uniform = [](const uint16_t* p) {
@@ -759,22 +759,36 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   };
   // First K step of slab kt (stage u): behind its MFMAs the fragments of the second step, and the last
   // loads of slab kt + 1.
-  auto step0 = [&](int u, int kt, bool next) {
+  // The waves leave every barrier together and run the same instructions, so a fragment read that follows the same
+  // MFMA in all of them is four 1 KB requests at once against an LDS that moves 128 bytes per cycle
+  // (SQ_LDS_CMD_FIFO_FULL counted the waves stalled at issue): the reads are spread over the whole step instead of
+  // following the step's first MFMAs in a row (+0.5 %).  Giving each wave its own load slot within a group of LEV
+  // MFMAs (one copy of the loop per wave) or holding wave w back by 16 w cycles behind the barrier measured -0.4 %
+  // and -3 %: the address unit's FIFO is not filled by the waves' coincidence.
+  auto step0 = [&](int u, int kt, bool next, auto slot) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
       mfma(0, m);
       __builtin_amdgcn_sched_barrier(0);
-      if (m < TN) read_b(1, m, u, 1);
+      if (m % TN == TN / 2 - 1 && m / TN < TN) read_b(1, m / TN, u, 1);   // one per row group
       if (m % TN == TN - 1) read_a(m / TN, u, 1);
-      if (m % LEV == LEV - 1 && L1 + m / LEV < L && next) load(L1 + m / LEV, u ^ 1, kt + 1);
+      if (L1 + m / LEV < L && next) {
+        if (m % LEV == decltype(slot)::value) load(L1 + m / LEV, u ^ 1, kt + 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   // Second K step: two row groups, the barrier, then behind the MFMAs the first-step fragments of slab
   // kt + 1 (other stage) and the first loads of slab kt + 2 into this stage.
-  auto step1 = [&](int u, int kt, bool next, bool next2) {
+  auto step1 = [&](int u, int kt, bool next, bool next2, auto slot) {
     __builtin_amdgcn_sched_barrier(0);
+    // Behind the barrier: the first-step fragments of slab kt + 1 (other stage).  Token fragments of the row groups
+    // that ran ahead of the barrier first, then one weight fragment every BSTEP MFMAs (the last one lands a dozen
+    // MFMAs before its first use), token fragments of the other groups as their last MFMA issues.
+    constexpr int G0 = BAR / TN;                        // row groups ahead of the barrier
+    constexpr int BSTEP = (NM - BAR - 2 * G0 - 2) / TN; // spacing of the weight-fragment reads
+    static_assert(BSTEP >= 1, "no room for the weight fragments behind the barrier");
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
       if (m == BAR) {
@@ -784,11 +798,14 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
       mfma(1, m);
       __builtin_amdgcn_sched_barrier(0);
       if (next) {
-        if (m >= BAR && m < BAR + BAR / TN) read_a(m - BAR, u ^ 1, 0);  // the groups that ran ahead of the barrier
-        else if (m >= BAR + BAR / TN && m < BAR + BAR / TN + TN) read_b(0, m - BAR - BAR / TN, u ^ 1, 0);
-        if (m > BAR + BAR / TN && m % TN == TN - 1) read_a(m / TN, u ^ 1, 0);
+        if (m >= BAR && m < BAR + 2 * G0 && (m - BAR) % 2 == 0) read_a((m - BAR) / 2, u ^ 1, 0);
+        if (m >= BAR + 2 * G0 && (m - BAR - 2 * G0) % BSTEP == 0 && (m - BAR - 2 * G0) / BSTEP < TN)
+          read_b(0, (m - BAR - 2 * G0) / BSTEP, u ^ 1, 0);
+        if (m / TN >= G0 && m % TN == TN - 1) read_a(m / TN, u ^ 1, 0);
       }
-      if (m >= BAR && (m - BAR) % LEV == LEV - 1 && (m - BAR) / LEV < L1 && next2) load((m - BAR) / LEV, u, kt + 2);
+      if (m >= BAR && (m - BAR) / LEV < L1 && next2) {
+        if ((m - BAR) % LEV == decltype(slot)::value) load((m - BAR) / LEV, u, kt + 2);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -809,18 +826,20 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   for (int i = 0; i < TM; ++i) read_a(i, 0, 0);
 
   int k0 = 0;
+  constexpr std::integral_constant<int, LEV - 1> slot{};  // every wave issues its load behind the last MFMA of a group of LEV
   for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches
-    step0(0, k0, true);
-    step1(0, k0, true, true);
-    step0(1, k0 + 1, true);
-    step1(1, k0 + 1, true, true);
+    step0(0, k0, true, slot);
+    step1(0, k0, true, true, slot);
+    step0(1, k0 + 1, true, slot);
+    step1(1, k0 + 1, true, true, slot);
   }
+  constexpr auto last_slot = slot;
   for (; k0 < nk; k0 += 2) {
-    step0(0, k0, k0 + 1 < nk);
-    step1(0, k0, k0 + 1 < nk, k0 + 2 < nk);
+    step0(0, k0, k0 + 1 < nk, last_slot);
+    step1(0, k0, k0 + 1 < nk, k0 + 2 < nk, last_slot);
     if (k0 + 1 < nk) {
-      step0(1, k0 + 1, k0 + 2 < nk);
-      step1(1, k0 + 1, k0 + 2 < nk, k0 + 3 < nk);
+      step0(1, k0 + 1, k0 + 2 < nk, last_slot);
+      step1(1, k0 + 1, k0 + 2 < nk, k0 + 3 < nk, last_slot);
     }
   }
   // The compiler does not see that the asm statements are matrix instructions: give the last of them the
