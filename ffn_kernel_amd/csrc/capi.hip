@@ -244,7 +244,7 @@ int linear_stream_splits(int64_t M, int64_t K, int64_t N) {
 RoutedPlan linear_plan(int64_t M, int64_t K, int64_t N) {
   RoutedPlan p = down_plan(M, N, K);
   if (N % 4 != 0) p.splits = 1;  // the reduce pass moves four columns per thread
-  if (p.splits == 1) p.tile = routed_tile(M, N, false);
+  if (p.splits == 1) p.tile = routed_tile(M, N, false, K);
   return p;
 }
 // fp32 partials of the tiled MaskedLinear forward: split-K for the whole GEMM, or the split tail of
@@ -499,7 +499,7 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
   RoutedPlan plan = linear_plan(M, K, N);
   if (!direct) {
     plan.splits = 1;
-    plan.tile = routed_tile(M, N, false);
+    plan.tile = routed_tile(M, N, false, K);
   }
   if (plan.splits > 1) {
     g.splits = plan.splits;

@@ -698,7 +698,10 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   constexpr int STAGE = Cfg::STAGE_BYTES, A_BYTES = Cfg::A_BYTES;
   constexpr int NM = TM * TN;
   constexpr int BAR = 2 * TN;            // MFMAs of a slab's second step ahead of the barrier (two row groups)
-  constexpr int LEV = 4;                 // one load behind every fourth MFMA
+  // One load per wave behind every LEV-th MFMA.  Four waves x one load per four MFMAs is the address unit's own rate
+  // (16 cycles per load and CU); the SwiGLU tile, whose two weight panels arrive from different matrices, measures
+  // 1.6 % faster a notch slower, the single-weight tiles 1-2.5 % slower.
+  constexpr int LEV = (NWAVES == 4 && Cfg::DUAL) ? 5 : 4;
   constexpr int L1 = (NM - BAR) / LEV;   // loads of the slab after next that go out in the second step
   static_assert(TM >= 3 && TM >= TN && L1 >= 1 && L1 <= L && (L - L1) * LEV <= NM, "schedule does not fit this wave tile");
   const int wave = tl.wave_s;

@@ -51,16 +51,19 @@ inline const TunedPlan* tuned_plan(int op, int64_t M, int64_t k, int64_t n) {
 
 // Routed GEMM over M rows and n_out output columns (K: the contraction, 0 = not known to the caller).
 inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual, int64_t K = 0, bool use_table = true) {
-  if (use_table && dual && K > 0)
-    if (const TunedPlan* t = tuned_plan(TUNED_DUAL, M, K, n_out)) return t->tile;
+  if (use_table && K > 0) {
+    if (const TunedPlan* t = tuned_plan(dual ? TUNED_DUAL : TUNED_PLAIN, M, K, n_out))
+      if (dual || t->splits == 1) return t->tile;
+  }
   auto tiles = [&](int tile) {
     const TileGeom t = tile_geom(tile, dual);
     return cdiv64(M, t.block_m) * cdiv64(n_out, t.block_n_out);
   };
   // At least two full rounds of 256x256 tiles.  The SwiGLU kernel runs them with four wavefronts of
-  // 128x128 (a third fewer LDS reads per flop; measured 4 % faster at M = 32768, d = 4096, h = 14336),
-  // the single-weight kernels with eight of 128x64 (the same time there, and less exposed when K is short).
-  if (tiles(TILE_256x256_W8) >= 2 * kCus) return dual ? TILE_256x256_W4 : TILE_256x256_W8;
+  // 128x128 (a third fewer LDS reads per flop; measured 4 % faster at M = 32768, d = 4096, h = 14336); so do the
+  // single-weight kernels over a long contraction (1-2.5 % faster at K = 4096 and 14336, N = 4096, M >= 16384),
+  // which otherwise keep eight wavefronts of 128x64 (less exposed when K is short).
+  if (tiles(TILE_256x256_W8) >= 2 * kCus) return dual || K >= 4096 ? TILE_256x256_W4 : TILE_256x256_W8;
   if (tiles(TILE_128x128_W4) >= kCus) return TILE_128x128_W4;
   return TILE_SMALL_W4;
 }
@@ -127,7 +130,7 @@ inline RoutedPlan pick_routed_plan(int64_t M, int64_t n_out, int64_t K, bool use
       p.splits = (K % 64 == 0 && M < 65536 && n_out % 4 == 0) ? t->splits : 1;
       return p;
     }
-  p.tile = pick_routed_tile(M, n_out, false);
+  p.tile = pick_routed_tile(M, n_out, false, K, use_table);
   p.splits = 1;
   if (M > 4096 || K % 64 != 0) return p;
   double best_cost = 0.0;
