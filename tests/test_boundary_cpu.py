@@ -224,3 +224,13 @@ def test_measured_plans_are_consulted_before_the_rules():
         finally:
             lib.ffnk_debug_force_tile(-1)
         assert isinstance(rules["split_k"], int)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """This build measures one GPU: bench.py --gpus N with N above 1 exits with a message, before it touches a device."""
+    import subprocess
+    import sys
+    bench = Path(__file__).resolve().parents[1] / "bench.py"
+    proc = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 2
+    assert "one GPU" in proc.stderr and not proc.stdout.strip()

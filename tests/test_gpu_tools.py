@@ -71,3 +71,32 @@ def test_forced_splits_results_match(dev):
             assert_close(MaskedLinear.apply(dw.x, dw.Wv.T, dw.Wt.T, dw.mask), ref, f"splits {s}")
     finally:
         lib.ffnk_debug_force_splits(-1)
+
+
+_BENCH = str(__import__("pathlib").Path(__file__).resolve().parents[1] / "bench.py")
+
+
+@pytest.mark.parametrize("workload", ["cfg2", "cfg3", "decode8"])
+def test_bench_prints_one_json_line_with_roofline_and_cpu_baseline(dev, workload):
+    """bench.py's contract on a short run: one JSON object, the headline fields, a roofline for the
+    dominant kernel and the CPU baseline of the same workload."""
+    import subprocess
+    import sys
+    note(f"bench.py --workload {workload}")
+    proc = subprocess.run([sys.executable, _BENCH, "--workload", workload, "--steps", "3", "--warmup", "1", "--cpu-rows", "64"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [l for l in proc.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in rec, key
+    assert rec["n_gpus"] == 1 and rec["steps"] == 3 and rec["warmup"] == 1 and rec["dtype"] == "bf16"
+    assert rec["value"] > 0 and rec["ms_per_step"] > 0 and "workload" in rec["config"]
+    roof = rec["roofline"]
+    assert roof["bound"] in ("mfma", "hbm") and roof["unit"] in ("TFLOP/s", "GB/s")
+    assert 0 < roof["frac"] < 1 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-9
+    assert roof["traffic"] is None or roof["traffic"] > 0
+    cpu = rec["cpu_baseline"]
+    assert cpu["value"] > 0 and cpu["cores"] >= 1 and cpu["kind"] == "port" and cpu["sample"]
