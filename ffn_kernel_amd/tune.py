@@ -21,6 +21,7 @@ geometric-mean time beats the baseline by more than --margin.
     python -m ffn_kernel_amd.tune                 # sweep, print the comparison
     python -m ffn_kernel_amd.tune --emit          # ... and rewrite csrc/tile_table_gen.hpp (then rebuild)
     python -m ffn_kernel_amd.tune --quick         # two buckets per layer (smoke test of the harness)
+    python -m ffn_kernel_amd.tune --ffn 5120,13824 --linear 5120,5120 --emit   # ... with a model's own layers added
 """
 from __future__ import annotations
 
@@ -43,8 +44,8 @@ GEN_PATH = Path(__file__).resolve().parent / "csrc" / "tile_table_gen.hpp"
 # M buckets [lo, hi]; each is measured at its upper end.  Below 65 rows the FFN runs the streaming kernels.
 BUCKETS = [(65, 128), (129, 256), (257, 512), (513, 1024), (1025, 2048), (2049, 4096), (4097, 8192), (8193, 16384),
            (16385, 32768)]
-FFN_LAYERS = [(1024, 2048), (4096, 14336)]      # (d, h): cfg2 and cfg4 / cfg5
-LINEAR_LAYERS = [(1024, 1024), (4096, 4096)]    # (K, N): cfg1 / cfg3 and an LLM-size projection
+FFN_LAYERS = [(1024, 2048), (2048, 8192), (4096, 14336)]    # (d, h): cfg2, a mid-size layer, cfg4 / cfg5
+LINEAR_LAYERS = [(1024, 1024), (2048, 2048), (4096, 4096)]  # (K, N): cfg1 / cfg3 and LLM-size projections
 
 
 class _Events:
@@ -346,7 +347,24 @@ def main(argv=None) -> int:
     ap.add_argument("--out", type=Path, default=GEN_PATH, help="where --emit writes")
     ap.add_argument("--json", default=None, help="dump every measurement")
     ap.add_argument("--quick", action="store_true", help="two buckets per layer")
+    ap.add_argument("--ffn", action="append", default=None, metavar="D,H",
+                    help="MaskedFFN layer to measure besides the default ones (repeatable)")
+    ap.add_argument("--linear", action="append", default=None, metavar="K,N",
+                    help="MaskedLinear layer to measure besides the default ones (repeatable)")
     args = ap.parse_args(argv)
+
+    def pairs(specs, default):
+        out = list(default)
+        for spec in specs or []:
+            a, b = (int(v) for v in spec.split(","))
+            if a <= 0 or b <= 0 or a % 8 or b % 8:
+                ap.error(f"layer extents must be positive multiples of 8, got {spec}")
+            if (a, b) not in out:
+                out.append((a, b))
+        return out
+
+    ffn_layers = pairs(args.ffn, FFN_LAYERS)
+    linear_layers = pairs(args.linear, LINEAR_LAYERS)
     if not torch.cuda.is_available():
         print("ffn_kernel_amd.tune needs a GPU", file=sys.stderr)
         return 2
@@ -359,7 +377,7 @@ def main(argv=None) -> int:
     def ratios(base, cand):
         return "  ".join(f"{k}:" + "/".join(f"{t / b_:.2f}" for t, b_ in zip(ts, base)) for k, ts in cand.items()) or "-"
 
-    for d, h in FFN_LAYERS:
+    for d, h in ffn_layers:
         for b in buckets:
             if b[1] * h * 2 > 4 << 30:
                 continue
@@ -370,7 +388,7 @@ def main(argv=None) -> int:
                   f"(tile {up['block_m']}x{up['block_n']}/{up['waves_m'] * up['waves_n']}w) down {_fmt_list(r['rules_down_ms'])}"
                   f" | up tile:ratio per scenario {ratios(r['rules_up_ms'], r['up_ms'])}"
                   f" | down (tile, splits):ratio {ratios(r['rules_down_ms'], r['down_ms'])}", flush=True)
-    for K, N in LINEAR_LAYERS:
+    for K, N in linear_layers:
         for b in buckets:
             r = tune_linear_fwd(K, N, b, args.trials, dev, args.margin)
             records.append(r)
