@@ -356,7 +356,10 @@ def main(argv=None) -> int:
     def pairs(specs, default):
         out = list(default)
         for spec in specs or []:
-            a, b = (int(v) for v in spec.split(","))
+            try:
+                a, b = (int(v) for v in spec.split(","))
+            except ValueError:
+                ap.error(f"expected two integers separated by a comma, got {spec}")
             if a <= 0 or b <= 0 or a % 8 or b % 8:
                 ap.error(f"layer extents must be positive multiples of 8, got {spec}")
             if (a, b) not in out:

@@ -234,3 +234,15 @@ def test_bench_refuses_more_than_one_gpu():
     proc = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 2
     assert "one GPU" in proc.stderr and not proc.stdout.strip()
+
+
+def test_tuner_checks_its_layer_arguments_before_it_needs_a_gpu():
+    """--ffn D,H / --linear K,N add layers to the sweep: extents that the MFMA paths cannot take are refused
+    at the command line; without a GPU the tuner then says so and returns 2."""
+    from ffn_kernel_amd import tune
+    with pytest.raises(SystemExit):
+        tune.main(["--ffn", "100,200"])
+    with pytest.raises(SystemExit):
+        tune.main(["--linear", "1024"])
+    if not torch.cuda.is_available():
+        assert tune.main(["--ffn", "2048,5632", "--linear", "2048,2048", "--quick"]) == 2
