@@ -23,6 +23,7 @@ _SIGNATURES = {
     "ffnk_debug_force_splits": (c_int, [c_int]),
     "ffnk_route": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "ffnk_workspace_bytes": (c_size_t, [c_int, c_int64, c_int64, c_int64]),
+    "ffnk_workspace_bytes_ffn_bwd": (c_size_t, [c_int64] * 9),
     "ffnk_tile_config": (c_int, [c_int, c_int64, c_int64, c_int64, c_void_p]),
     "ffnk_masked_linear_fwd": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p,
                                        c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_size_t,

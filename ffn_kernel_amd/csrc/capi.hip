@@ -119,25 +119,49 @@ constexpr int kBwdPadRows = 64;
 struct FfnBwdPlan {
   BwdPlan up, dn;  // weight-gradient GEMM shapes: up = dW1/dW3 (K = d, N = h), dn = dW2 (K = h, N = d)
   int64_t ldt;
+  size_t w2t_bytes;  // room at off_w2t: the W2^T / U2^T copies, or the dx GEMM's partials / split tail after them
   size_t off_t13, off_dh, off_w2t, off_w13t, off_gt, off_xt, off_ht, off_d1t, off_d3t, off_p, total;
 };
-FfnBwdPlan plan_ffn_bwd(int64_t M, int64_t d, int64_t h, bool dup_k_contig, bool ddn_k_contig) {
+// Which of the optional regions a call touches (decided from strides and alignment, the same way by the
+// planner and by the backward itself): copies of the down / up weights for layouts the K-major kernels do not
+// read in place, and transposes of H, dt1, dt3 when their rows do not fit 32-bit slab offsets.
+struct FfnBwdPaths {
+  bool w2_copy = true, w13_copy = true, acts_in_place = false, dx_direct = false;
+};
+constexpr FfnBwdPaths kFfnBwdWorstCase{};
+// Weight-gradient split of the in-place path (H, dt1, dt3 read where they lie).
+TileChoice ffn_bwd_in_place_choice(int64_t M, int64_t d, int64_t h) {
+  TileChoice tc = pick_splitk_tile(M, h, d, use_tuned());
+  if (forced_splits() >= 1) tc.splits = forced_splits();
+  return tc;
+}
+// Tile and split of the dx GEMM (2h-long contraction) and the bytes of partials or split tail it wants.
+RoutedPlan ffn_bwd_dx_plan(int64_t M, int64_t d, int64_t h, bool dx_direct, size_t room, size_t* need);
+FfnBwdPlan plan_ffn_bwd(int64_t M, int64_t d, int64_t h, bool dup_k_contig, bool ddn_k_contig,
+                        const FfnBwdPaths& paths = kFfnBwdWorstCase) {
   FfnBwdPlan p;
   p.up = plan_bwd(M, d, h, dup_k_contig);
   p.dn = plan_bwd(M, h, d, ddn_k_contig);
   p.ldt = padded_rows(M);
-  const int splits = p.up.tc.splits > p.dn.tc.splits ? p.up.tc.splits : p.dn.tc.splits;
+  int splits = p.up.tc.splits > p.dn.tc.splits ? p.up.tc.splits : p.dn.tc.splits;
+  if (paths.acts_in_place) splits = ffn_bwd_in_place_choice(M, d, h).splits;
+  const size_t w2_copies = 2 * ws_align((size_t)h * d * 2);
+  // The dx GEMM's partials (or split tail) live where the copies would, as far as they fit there - the same bound
+  // whether or not the copies are made, so that the dx GEMM's plan does not depend on the layout.
+  size_t dx_need = 0;
+  ffn_bwd_dx_plan(M, d, h, paths.dx_direct, w2_copies, &dx_need);
+  p.w2t_bytes = paths.w2_copy ? w2_copies : ws_align(dx_need);
   size_t o = route_ws_bytes(M);
   p.off_t13 = o;  o += ws_align((size_t)(M + kBwdPadRows) * 2 * h * 2);
   p.off_dh = o;   o += ws_align((size_t)(M + kBwdPadRows) * h * 2);
-  p.off_w2t = o;  o += 2 * ws_align((size_t)h * d * 2);
-  p.off_w13t = o; o += 2 * ws_align((size_t)d * 2 * h * 2);
+  p.off_w2t = o;  o += p.w2t_bytes;
+  p.off_w13t = o; o += paths.w13_copy ? 2 * ws_align((size_t)d * 2 * h * 2) : 0;
   p.off_gt = o;   o += ws_align((size_t)d * p.ldt * 2);
   p.off_xt = o;   o += ws_align((size_t)d * p.ldt * 2);
-  p.off_ht = o;   o += ws_align((size_t)h * p.ldt * 2);
-  p.off_d1t = o;  o += ws_align((size_t)h * p.ldt * 2);
-  p.off_d3t = o;  o += ws_align((size_t)h * p.ldt * 2);
-  p.off_p = o;    o += ws_align((size_t)2 * splits * d * h * 4);
+  p.off_ht = o;   o += paths.acts_in_place ? 0 : ws_align((size_t)h * p.ldt * 2);
+  p.off_d1t = o;  o += paths.acts_in_place ? 0 : ws_align((size_t)h * p.ldt * 2);
+  p.off_d3t = o;  o += paths.acts_in_place ? 0 : ws_align((size_t)h * p.ldt * 2);
+  p.off_p = o;    o += (paths.acts_in_place && splits == 1) ? 0 : ws_align((size_t)2 * splits * d * h * 4);
   p.total = o;
   return p;
 }
@@ -228,6 +252,47 @@ RoutedPlan down_plan(int64_t M, int64_t d, int64_t h) {
     p.splits = fs;
   return p;
 }
+// dx GEMM of the MaskedFFN backward: few output tiles over a 2h-long contraction, so K is split like the forward's
+// down projection when the fp32 partials fit `room`; an unsplit big tile wants room for its split tail instead.
+RoutedPlan ffn_bwd_dx_plan(int64_t M, int64_t d, int64_t h, bool dx_direct, size_t room, size_t* need) {
+  RoutedPlan dxp = down_plan(M, d, 2 * h);
+  if (!dx_direct || (size_t)dxp.splits * M * d * 4 > room) {
+    dxp.splits = 1;
+    dxp.tile = routed_tile(M, d, false);
+  }
+  size_t n = 0;
+  if (dxp.splits > 1) n = (size_t)dxp.splits * M * d * 4;
+  else if (dx_direct && is_big_tile(dxp.tile) && (size_t)kTailSlots * 256 * 256 * 4 <= room) n = (size_t)kTailSlots * 256 * 256 * 4;
+  if (need) *need = n;
+  return dxp;
+}
+// Paths of the MaskedFFN backward for one layout: which weights are read in place and which copied, and whether
+// H, dt1, dt3 are read in place by the weight-gradient GEMMs.  The backward and the lean workspace query both ask
+// here, so that the regions a call touches are the regions its plan holds.
+FfnBwdPaths ffn_bwd_paths(int64_t M, int64_t d, int64_t h, int64_t g_stride_m, int64_t up_stride_n, int64_t down_stride_k,
+                          int64_t down_stride_n, const uint16_t* W1, const uint16_t* W3, const uint16_t* U1,
+                          const uint16_t* U3, const uint16_t* W2, const uint16_t* U2, bool* w2_direct_out = nullptr,
+                          bool* w2_kmajor_out = nullptr, bool* w13_kmajor_out = nullptr) {
+  const int64_t ld13 = 2 * h;
+  const bool w2_direct = down_stride_n == 1 && down_stride_k % 8 == 0 && down_stride_k >= d && aligned16(W2) && aligned16(U2);
+  // The forward's layout ([d, h] rows, h contiguous) is K-major for the dh GEMM: read in place.
+  const bool w2_kmajor = !w2_direct && down_stride_k == 1 && kmajor_ok(d, h, down_stride_n, W2, U2) &&
+                         direct_ok(d, M, g_stride_m, 8);
+  // The up-projection weights ([h, d] rows, d contiguous) are K-major for the dx GEMM: the contraction
+  // runs through the gate weight's rows and on into the up weight's.
+  const bool w13_kmajor = h % 64 == 0 && kmajor_ok(2 * h, d, up_stride_n, W1, W3) && aligned16(U1) && aligned16(U3) &&
+                          direct_ok(2 * h, 0, ld13, 8);
+  FfnBwdPaths paths;
+  paths.w2_copy = !(w2_direct || w2_kmajor);
+  paths.w13_copy = !w13_kmajor;
+  paths.acts_in_place = ld13 * 128 + 2 * h < ((int64_t)1 << 32);
+  paths.dx_direct = w13_kmajor || direct_ok(2 * h, 0, ld13, ld13);
+  if (w2_direct_out) *w2_direct_out = w2_direct;
+  if (w2_kmajor_out) *w2_kmajor_out = w2_kmajor;
+  if (w13_kmajor_out) *w13_kmajor_out = w13_kmajor;
+  return paths;
+}
+
 // MaskedLinear forward at decode sizes: 0 = LDS-tiled GEMM, 1 = dot-product streams (M <= 8),
 // 2 = LDS-transposed streams (M <= 64).  The op is bound by reading each weight once.
 int linear_stream_kind(int64_t M, int64_t K, int64_t N) {
@@ -351,6 +416,15 @@ size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N) {
     default:
       return (size_t)-1;
   }
+}
+
+size_t ffnk_workspace_bytes_ffn_bwd(int64_t M, int64_t d, int64_t h, int64_t g_stride_m, int64_t up_stride_n,
+                                    int64_t down_stride_k, int64_t down_stride_n, int64_t dup_stride_k,
+                                    int64_t ddown_stride_k) {
+  if (M < 0 || d <= 0 || h <= 0 || M > kMaxRows || d > kMaxCols || h > kMaxCols) return (size_t)-1;
+  const FfnBwdPaths paths = ffn_bwd_paths(M, d, h, g_stride_m, up_stride_n, down_stride_k, down_stride_n, nullptr, nullptr,
+                                          nullptr, nullptr, nullptr, nullptr);
+  return plan_ffn_bwd(M, d, h, dup_stride_k == 1, ddown_stride_k == 1, paths).total;
 }
 
 int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t* out) {
@@ -819,14 +893,20 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   if (!ok)
     return fail(FFNK_E_STRIDE, "MaskedFFN backward: d, h and the row strides must be multiples of 8, rows 16-byte "
                                "aligned and the up-projection weights K-contiguous (up_stride_k == 1)");
-  const FfnBwdPlan p = plan_ffn_bwd(M, d, h, dup_stride_k == 1, ddown_stride_k == 1);
-  if (ws_bytes < p.total || !ws) return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, p.total);
+  // Which optional regions this layout needs (ffnk_workspace_bytes_ffn_bwd asks the same function).
+  const int64_t ld13 = 2 * h;
+  bool w2_direct = false, w2_kmajor = false, w13_kmajor = false;
+  const FfnBwdPaths paths = ffn_bwd_paths(M, d, h, g_stride_m, up_stride_n, down_stride_k, down_stride_n, W1, W3, U1, U3, W2,
+                                          U2, &w2_direct, &w2_kmajor, &w13_kmajor);
+  const FfnBwdPlan p = plan_ffn_bwd(M, d, h, dup_stride_k == 1, ddown_stride_k == 1, paths);
+  if (ws_bytes < p.total || !ws)
+    return fail(FFNK_E_WORKSPACE, "workspace %zu < %zu bytes (ffnk_workspace_bytes_ffn_bwd sizes it for aligned pointers; "
+                                  "ffnk_workspace_bytes(FFNK_OP_FFN_BWD) for any layout)", ws_bytes, p.total);
   if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
   uint8_t* wsb = static_cast<uint8_t*>(ws);
   const RouteWs r = carve_route(wsb, M);
   uint16_t* T13 = reinterpret_cast<uint16_t*>(wsb + p.off_t13);
   uint16_t* DH = reinterpret_cast<uint16_t*>(wsb + p.off_dh);
-  const int64_t ld13 = 2 * h;
   FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
 
   // ---- pre-activations, routed order: T13[:, 0:h] = x A1, T13[:, h:2h] = x A3 ----
@@ -846,10 +926,6 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   // ---- dh = gather(g) @ A2^T: contraction over d needs the down weights as [h, d] rows ----
   const uint16_t* w2t[2] = {W2, U2};
   int64_t ld2 = down_stride_k;
-  const bool w2_direct = down_stride_n == 1 && down_stride_k % 8 == 0 && down_stride_k >= d && aligned16(W2) && aligned16(U2);
-  // The forward's layout ([d, h] rows, h contiguous) is K-major for this GEMM: read in place.
-  const bool w2_kmajor = !w2_direct && down_stride_k == 1 && kmajor_ok(d, h, down_stride_n, W2, U2) &&
-                         direct_ok(d, M, g_stride_m, 8);
   if (w2_kmajor) {
     ld2 = down_stride_n;
   } else if (!w2_direct) {
@@ -869,11 +945,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
            "SwiGLU backward pass");
 
   // ---- dx = (dt1 | dt3) @ (A1^T | A3^T)^T: one GEMM over the concatenated contraction of length 2h ----
-  // The up-projection weights ([h, d] rows, d contiguous) are K-major for this GEMM: the contraction
-  // runs through the gate weight's rows and on into the up weight's.  Otherwise both are copied
-  // into one [d, 2h] operand per modality.
-  const bool w13_kmajor = h % 64 == 0 && kmajor_ok(2 * h, d, up_stride_n, W1, W3) && aligned16(U1) && aligned16(U3) &&
-                          direct_ok(2 * h, 0, ld13, 8);
+  // In place over the K-major up-projection weights, or over one [d, 2h] copy per modality.
   GemmArgs b;
   b.A = T13; b.lda = ld13;
   if (w13_kmajor) {
@@ -892,17 +964,14 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   b.M = (int)M; b.N = (int)d; b.K = (int)(2 * h);
   // Few output tiles over a 2h-long contraction: split K like the forward's down projection.  The
   // fp32 partials live where the W2^T copies were (dead since the dh GEMM), if they fit there.
-  const bool dx_direct = w13_kmajor || direct_ok(2 * h, 0, ld13, ld13);
-  RoutedPlan dxp = down_plan(M, d, 2 * h);
-  if (!dx_direct || (size_t)dxp.splits * M * d * 4 > 2 * ws_align((size_t)h * d * 2)) {
-    dxp.splits = 1;
-    dxp.tile = routed_tile(M, d, false);
-  }
+  const bool dx_direct = paths.dx_direct;
+  size_t dx_need = 0;
+  const RoutedPlan dxp = ffn_bwd_dx_plan(M, d, h, dx_direct, 2 * ws_align((size_t)h * d * 2), &dx_need);
+  if (dx_need > p.w2t_bytes) return fail(FFNK_E_WORKSPACE, "internal: dx partials %zu > %zu planned", dx_need, p.w2t_bytes);
   if (dxp.splits > 1) {
     b.splits = dxp.splits;
     b.P = reinterpret_cast<float*>(wsb + p.off_w2t);
-  } else if (dx_direct && is_big_tile(dxp.tile) &&
-             (size_t)kTailSlots * 256 * 256 * 4 <= 2 * ws_align((size_t)h * d * 2)) {
+  } else if (dx_need > 0) {
     b.P_tail = reinterpret_cast<float*>(wsb + p.off_w2t);  // split tail of the last, partial round
   }
   if (w13_kmajor) FFNK_HIP(launch_down_gemm_kmajor(dxp.tile, b, stream), "dx GEMM");
@@ -916,12 +985,11 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);    // [d, ldt]
   uint16_t* XT = reinterpret_cast<uint16_t*>(wsb + p.off_xt);    // [d, ldt]
   float* P = reinterpret_cast<float*>(wsb + p.off_p);
-  const bool in_place = ld13 * 128 + 2 * h < ((int64_t)1 << 32);
+  const bool in_place = paths.acts_in_place;
   if (in_place) {
     FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, x, x_stride_m, (int)d, XT, p.ldt, r.perm, r.counts, (int)M,
                                       stream, false, false), "g / x transpose");
-    TileChoice tc = pick_splitk_tile(M, h, d, use_tuned());
-    if (forced_splits() >= 1) tc.splits = forced_splits();
+    const TileChoice tc = ffn_bwd_in_place_choice(M, d, h);
     const int tile = forced_tile() >= 0 ? forced_tile() : tc.tile;
     // out[r * sr + c * sc]: r runs over h (the in-place operand's columns), c over d
     auto weight_grad_in_place = [&](const uint16_t* rows, int64_t ld_rows, const uint16_t* cT, uint16_t* o0, uint16_t* o1,

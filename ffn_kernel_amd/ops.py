@@ -266,7 +266,14 @@ def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None):
     gdsk, gdsn = _wstrides(ddowns[0])
     lib = _lib.load()
     with _on_device(dev):
-        ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
+        # Sized for this layout when every weight is 16-byte aligned (what the lean query assumes), for any
+        # layout otherwise: the usual views then skip the room for weight copies and transposed intermediates.
+        if all(w.data_ptr() % 16 == 0 for w in (*ups, *downs)):
+            ws_bytes = lib.ffnk_workspace_bytes_ffn_bwd(M, d, h, grad.stride(0) if M > 1 else d, usn, dsk, dsn, gusk, gdsk)
+            if ws_bytes == (1 << 64) - 1:
+                raise ValueError(f"ffnk_workspace_bytes_ffn_bwd: invalid extents M={M} d={d} h={h}")
+        else:
+            ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
         head = (grad.data_ptr(), grad.stride(0) if M > 1 else d, a.data_ptr(), a.stride(0) if M > 1 else d,
                 ups[0].data_ptr(), ups[1].data_ptr(), ups[2].data_ptr(), ups[3].data_ptr(), usk, usn,

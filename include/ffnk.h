@@ -97,6 +97,17 @@ FFNK_API int ffnk_route(const uint8_t* mask, int64_t M, int32_t* perm, int32_t* 
  * Returns (size_t)-1 for an unknown op or invalid extents. */
 FFNK_API size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N);
 
+/* Scratch of ffnk_masked_ffn_bwd / ffnk_masked_ffn_bwd_saved for one layout of the weights (element strides as
+ * passed to those calls), assuming 16-byte aligned pointers.  ffnk_workspace_bytes(FFNK_OP_FFN_BWD, ...) covers every
+ * layout and reserves room for copies of the weights and transposes of the intermediates that the usual layout
+ * (nn.Linear.weight.T views, d and h multiples of 64) never touches - 1.6 GB of 2.7 GB at M = 8192, d = 4096,
+ * h = 14336; this query leaves that out.  A call whose pointers turn out not to be aligned needs the larger size
+ * and says so (FFNK_E_WORKSPACE).  No counterpart in the reference, whose MaskedFFN.backward raises
+ * (ffn_kernel/ops.py:34-38).  Returns (size_t)-1 for invalid extents. */
+FFNK_API size_t ffnk_workspace_bytes_ffn_bwd(int64_t M, int64_t d, int64_t h, int64_t g_stride_m, int64_t up_stride_n,
+                                             int64_t down_stride_k, int64_t down_stride_n, int64_t dup_stride_k,
+                                             int64_t ddown_stride_k);
+
 /* Which tile-table entry the library uses for these extents. */
 FFNK_API int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t* out);
 

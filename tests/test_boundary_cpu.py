@@ -246,3 +246,15 @@ def test_tuner_checks_its_layer_arguments_before_it_needs_a_gpu():
         tune.main(["--linear", "1024"])
     if not torch.cuda.is_available():
         assert tune.main(["--ffn", "2048,5632", "--linear", "2048,2048", "--quick"]) == 2
+
+
+def test_lean_ffn_backward_workspace_never_exceeds_the_any_layout_one():
+    lib = _lib.load()
+    for M, d, h in ((0, 64, 64), (1, 64, 128), (300, 256, 512), (4096, 4096, 14336), (8192, 4096, 14336), (333, 72, 200)):
+        worst = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
+        for usn, dsk, dsn in ((d, 1, h), (d, d, 1), (d + 8, 1, h + 8), (d, 3, h)):
+            for gk in (1, h):
+                lean = lib.ffnk_workspace_bytes_ffn_bwd(M, d, h, d, usn, dsk, dsn, gk, gk)
+                assert 0 < lean <= worst, (M, d, h, usn, dsk, dsn, gk, lean, worst)
+    assert lib.ffnk_workspace_bytes_ffn_bwd(8192, 4096, 14336, 4096, 4096, 1, 14336, 1, 1) < 1 << 30
+    assert lib.ffnk_workspace_bytes_ffn_bwd(-1, 64, 64, 64, 64, 1, 64, 1, 1) == ctypes.c_size_t(-1).value

@@ -877,3 +877,48 @@ def test_linear_bwd_fused_launch(dev, M, K, N, p):
     again = masked_linear_backward(d.grad, d.x, d.Wv.T, d.Wt.T, d.mask)
     for a, b in zip((dx, dWv, dWt), again):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("M,d,h,layout", [(300, 256, 512, "views"), (2100, 512, 1024, "views"), (4100, 256, 1024, "views"),
+                                          (300, 256, 512, "down_contig"), (333, 72, 200, "views"),
+                                          (500, 128, 96, "views")])
+def test_ffn_bwd_lean_workspace_is_enough_and_changes_nothing(dev, M, d, h, layout, monkeypatch):
+    """The backward sizes its workspace for the layout at hand (ffnk_workspace_bytes_ffn_bwd): never more than the
+    any-layout size, nothing written past its end (guard bytes behind it stay intact), and gradients bit-identical
+    to a run on the any-layout workspace."""
+    from ffn_kernel_amd import ops
+    note(f"ffn bwd lean workspace M={M} d={d} h={h} {layout}")
+    gen = torch.Generator().manual_seed(M + d)
+    mask = (torch.rand(M, generator=gen) < 0.5).to(dev)
+    w = wl.make_ffn("t", M, d, h, mask.cpu(), seed=M + 7, w_std=0.05).to(dev)
+    g = torch.randn(M, d, generator=gen).to(torch.bfloat16).to(dev)
+    Wt = {k: v.T for k, v in w.W.items()}
+    if layout == "down_contig":
+        Wt["w2"], Wt["u2"] = Wt["w2"].contiguous(), Wt["u2"].contiguous()
+    args = (g, w.x, Wt["w1"], Wt["w2"], Wt["w3"], Wt["u1"], Wt["u2"], Wt["u3"], mask)
+    sizes, guards = [], []
+    real_workspace = ops._workspace
+
+    def guarded(nbytes, device):
+        t = torch.empty(max(nbytes, 16) + 4096, dtype=torch.uint8, device=device)
+        t[max(nbytes, 16):] = 0xA5
+        sizes.append(nbytes)
+        guards.append(t)
+        return t[:max(nbytes, 16)]
+
+    monkeypatch.setattr(ops, "_workspace", guarded)
+    lean = ops.masked_ffn_backward(*args)
+    torch.cuda.synchronize()
+    worst = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
+    assert len(sizes) == 1 and sizes[0] <= worst
+    assert bool((guards[0][max(sizes[0], 16):] == 0xA5).all()), "the backward wrote past its workspace"
+    # the same call on the any-layout workspace
+    monkeypatch.setattr(ops, "_workspace", real_workspace)
+    lib = _lib.load()
+    monkeypatch.setattr(lib, "ffnk_workspace_bytes_ffn_bwd", lambda *a: worst, raising=False)
+    ref = ops.masked_ffn_backward(*args)
+    torch.cuda.synchronize()
+    for a, b, name in zip(lean, ref, ("da", "dw1", "dw2", "dw3", "du1", "du2", "du3")):
+        assert torch.equal(a, b), name
+    if d % 64 == 0 and h % 64 == 0:
+        assert sizes[0] < worst  # weights and intermediates read in place: no room for copies or transposes
