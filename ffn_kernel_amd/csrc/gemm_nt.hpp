@@ -115,6 +115,12 @@ struct RoutedGemmCfg {
   // and written per 16 K-products of a lane instead of sixteen per 16: the kernel runs at the board's
   // power limit and the narrower accumulator traffic is worth 5 % there); the others with 32x32x16.
   static constexpr bool MFMA16 = DIRECT_ && !B_KMAJOR_ && BM_ == 256;
+  // Cache policy of the token panel's global->LDS loads.  The down projection's token rows (the routed intermediate,
+  // read in place) pass each XCD once: a round of tiles reads a line and no later round does.  Loaded with the
+  // non-temporal hint they do not push the weight panels out of L2 (cfg4 down projection 2.91 -> 2.85 ms, M = 16384
+  // 1.47 -> 1.45 ms; no measurable difference on the smaller tiles, which keep the default).  Gathered token rows
+  // are read again by the next rounds (the hint costs 9 % there), and so are the weights (2-4 %).
+  static constexpr int AUX_A = (MFMA16 && !GATHER_A_ && SCATTER_C_) ? 2 : 0;
   static constexpr int MT = MFMA16 ? 16 : 32;              // edge of an accumulator tile
   static constexpr int ACC_N = MT * MT / kWave;            // accumulator registers per tile
   using Acc = std::conditional_t<MFMA16, f32x4_t, f32x16_t>;
@@ -550,7 +556,7 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l - NJB], FFNK_LDS_PTR(st + ((l - NJB) * NWAVES + wave) * 1024), 16,
-                                               offA[l - NJB], ko, 0, 0);
+                                               offA[l - NJB], ko, 0, Cfg::AUX_A);
   };
   // One K step: MFMAs on fragment buffer `cur`; behind them the reads of (stage_next, step_next) into the
   // other buffer and loads [l0, l0 + FH) of slab kt_dma into stage_dma.
@@ -746,7 +752,7 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l - NJB], FFNK_LDS_PTR(st + ((l - NJB) * NWAVES + wave) * 1024), 16,
-                                               offA[l - NJB], ko, 0, 0);
+                                               offA[l - NJB], ko, 0, Cfg::AUX_A);
   };
   // Four-wave tiles hold 256 accumulator registers per lane, which only fit the accumulation half of the
   // register file.  Left to the builtin, the compiler keeps part of them in ordinary registers and moves
@@ -939,7 +945,7 @@ __device__ __forceinline__ void gemm_mainloop_ring(const TileLanes<Cfg>& tl,
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l - NJB], FFNK_LDS_PTR(st + ((l - NJB) * NWAVES + wave) * 1024), 16,
-                                               offA[l - NJB], ko, 0, 0);
+                                               offA[l - NJB], ko, 0, Cfg::AUX_A);
   };
   // One K step: the MFMAs on fragment buffer `cur`; behind them the fragment reads of (stage_next, ks_next)
   // into the other buffer and loads [l0, l0 + LQ) of slab kt_dma into stage_dma.
