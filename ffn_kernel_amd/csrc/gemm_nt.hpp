@@ -681,11 +681,14 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
 //    fragment of a group (16 rows x 32 K) is single-buffered and re-read in place for the next step as
 //    soon as the group's last MFMA has issued (a whole step ahead of its next use); the TN weight
 //    fragments are double-buffered and read during the previous step, one behind the middle MFMA of each row group.
-//  * One barrier per slab, behind the first two row groups of the slab's second step: by then every
-//    fragment read of the stage has returned (the last one was issued two groups earlier) and the next
-//    slab, whose last loads went out more than half a slab before, has landed.
-//  * The global->LDS loads go out at the rate the address unit takes them, one 1 KB load per wave
-//    behind every fourth MFMA (16 cycles per load and CU), not in a burst behind the barrier: the
+//  * Two barriers per slab, both in its second step.  The release barrier, behind the step's first four
+//    MFMAs: the stage's last fragment reads were issued at the end of the first step and have returned
+//    (lgkmcnt only), so the stage is free for the slab after next.  The data barrier, behind the first two
+//    row groups: the next slab has landed in the other stage (vmcnt leaves the loads issued since the
+//    release barrier in flight).  One barrier doing both jobs started the loads twelve MFMAs later (1-3 % slower;
+//    the waves run in step, a barrier by itself measures nothing).
+//  * The global->LDS loads go out no faster than the address unit takes them, one 1 KB load per wave
+//    behind every fourth or fifth MFMA (16 cycles per load and CU), not in a burst behind the barrier: the
 //    first loads of the slab after next through the rest of the second step, the others during the
 //    first step of the following slab - at least half a slab ahead of the barrier that waits for them.
 // =============================================================================================
@@ -703,12 +706,15 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   constexpr int L = NJA + NJB;
   constexpr int STAGE = Cfg::STAGE_BYTES, A_BYTES = Cfg::A_BYTES;
   constexpr int NM = TM * TN;
-  constexpr int BAR = 2 * TN;            // MFMAs of a slab's second step ahead of the barrier (two row groups)
-  // One load per wave behind every LEV-th MFMA.  Four waves x one load per four MFMAs is the address unit's own rate
-  // (16 cycles per load and CU); the SwiGLU tile, whose two weight panels arrive from different matrices, measures
-  // 1.6 % faster a notch slower, the single-weight tiles 1-2.5 % slower.
-  constexpr int LEV = (NWAVES == 4 && Cfg::DUAL) ? 5 : 4;
-  constexpr int L1 = (NM - BAR) / LEV;   // loads of the slab after next that go out in the second step
+  constexpr int BAR = 2 * TN;            // MFMAs of a slab's second step ahead of the data barrier (two row groups)
+  constexpr int RPOS = 4;                // ... ahead of the release barrier
+  // One load per wave behind every LEV-th MFMA.  One per four MFMAs is the address unit's own rate (16 cycles per
+  // load and CU).  The four-wave tiles measure faster a notch slower (SwiGLU tile 3 %, down projection 2.4 %, the
+  // gathered single-weight GEMM the same either way), the eight-wave tile 1-4 % slower; six is no better than five.
+  constexpr int LEV = NWAVES == 4 ? 5 : 4;
+  constexpr int L1 = (NM - RPOS) / LEV < L ? (NM - RPOS) / LEV : L;  // loads of the slab after next that go out in the second step
+  constexpr int NPRE = (BAR - RPOS) / LEV;  // ... of them ahead of the data barrier (a load follows the last MFMA of its group of LEV)
+  static_assert(RPOS >= 0 && RPOS < BAR && NPRE <= L1, "release barrier ahead of the data barrier");
   static_assert(TM >= 3 && TM >= TN && L1 >= 1 && L1 <= L && (L - L1) * LEV <= NM, "schedule does not fit this wave tile");
   const int wave = tl.wave_s;
 
@@ -800,8 +806,13 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
     static_assert(BSTEP >= 1, "no room for the weight fragments behind the barrier");
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
+      if (m == RPOS) {
+        dma_wait_barrier<63>();  // every wave's reads of stage u have returned: the stage is free for slab kt + 2
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (m == BAR) {
-        dma_wait_barrier<0>();
+        if (next2) dma_wait_barrier<NPRE>();  // slab kt + 1 has landed; the loads of slab kt + 2 issued since stay in flight
+        else dma_wait_barrier<0>();
         __builtin_amdgcn_sched_barrier(0);
       }
       mfma(1, m);
@@ -812,8 +823,8 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
           read_b(0, (m - BAR - 2 * G0) / BSTEP, u ^ 1, 0);
         if (m / TN >= G0 && m % TN == TN - 1) read_a(m / TN, u ^ 1, 0);
       }
-      if (m >= BAR && (m - BAR) / LEV < L1 && next2) {
-        if ((m - BAR) % LEV == decltype(slot)::value) load((m - BAR) / LEV, u, kt + 2);
+      if (m >= RPOS && (m - RPOS) / LEV < L1 && next2) {
+        if ((m - RPOS) % LEV == decltype(slot)::value) load((m - RPOS) / LEV, u, kt + 2);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
