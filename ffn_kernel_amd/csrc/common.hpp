@@ -28,7 +28,10 @@ __device__ __forceinline__ float bf2f(uint16_t v) {
 
 // Two fp32 -> packed pair of bf16 (lo in bits 0..15).
 __device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
-  return static_cast<uint32_t>(f2bf(lo)) | (static_cast<uint32_t>(f2bf(hi)) << 16);
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));  // one v_cvt_pk_bf16_f32
 }
 
 // silu(g) * u in fp32: g * sigmoid(g) * u.

@@ -1050,6 +1050,40 @@ template <class Cfg>
 __device__ __forceinline__ void routed_epilogue(const GemmArgs& g, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN], int row0,
                                                 int row_end, int n0, int wm, int wn, uint32_t lr, uint32_t lh) {
   constexpr int TM = Cfg::TM, TN_OUT = Cfg::TN_OUT, MT = Cfg::MT, RUNS = Cfg::ACC_N / 4;
+  // A tile inside the matrix on every side, with 8-byte aligned runs: no guards, one row pointer per row group and
+  // the column of every store an immediate offset.  (The guarded form below costs a compare and two branches per
+  // run of four outputs - as many cycles as the SwiGLU itself.)
+  const bool inside = row0 + Cfg::BM <= row_end && n0 + Cfg::BN_OUT <= g.N && (reinterpret_cast<uintptr_t>(g.C) & 7) == 0 &&
+                      (g.ldc & 3) == 0 && !(Cfg::DUAL && g.C_pre != nullptr);
+  if (inside) {
+    int64_t dst[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int p = row0 + wm * Cfg::WTM + i * MT + (int)lr;
+      dst[i] = Cfg::SCATTER_C ? (int64_t)g.perm[p] : (int64_t)p;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      uint16_t* crow = g.C + dst[i] * g.ldc + (n0 + wn * Cfg::WTN_OUT + acc_col<Cfg>(0, (int)lh));
+#pragma unroll
+      for (int j = 0; j < TN_OUT; ++j) {
+#pragma unroll
+        for (int q4 = 0; q4 < RUNS; ++q4) {
+          float o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (Cfg::DUAL) o[e] = swiglu(acc[i][j][4 * q4 + e], acc[i][j + TN_OUT][4 * q4 + e]);
+            else o[e] = acc[i][j][4 * q4 + e];
+          }
+          uint2 v2;
+          v2.x = pack2bf(o[0], o[1]);
+          v2.y = pack2bf(o[2], o[3]);
+          *reinterpret_cast<uint2*>(crow + j * MT + (acc_col<Cfg>(4 * q4, 0) - acc_col<Cfg>(0, 0))) = v2;
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int p = row0 + wm * Cfg::WTM + i * MT + (int)lr;
