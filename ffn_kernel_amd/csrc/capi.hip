@@ -448,6 +448,8 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
     }
     default: return fail(FFNK_E_OP, "unknown op %d", op);
   }
+  const bool direct = contraction > 0 && contraction % 64 == 0;
+  if (!direct && tile == TILE_256x256_W4) tile = TILE_256x256_W8;  // the four-wave tile runs on the direct path only
   const TileGeom gm = tile_geom(tile, dual);
   const bool stream = (op == FFNK_OP_FFN_FWD || op == FFNK_OP_FFN_UP || op == FFNK_OP_FFN_DOWN) && use_stream_path(M, K, N);
   out->path = stream ? FFNK_PATH_STREAM : FFNK_PATH_MFMA_TILED;
@@ -458,7 +460,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->waves_n = gm.waves_n;
   out->group_m = dual ? 8 : 4;
   out->split_k = splits;
-  out->direct_lds = (contraction > 0 && contraction % 64 == 0) ? 1 : 0;
+  out->direct_lds = direct ? 1 : 0;
   out->lds_stages = (tile == TILE_128x128_R4 && out->direct_lds) ? 4 : 2;
   if (op == FFNK_OP_FFN_DOWN && !stream) out->split_k = tiled_down_splits(M, K, N);
   if (op == FFNK_OP_LINEAR_FWD && linear_stream_kind(M, K, N)) {

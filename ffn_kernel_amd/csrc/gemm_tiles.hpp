@@ -43,7 +43,12 @@ template <class Tiles>
 inline hipError_t dispatch_tile(int tile, const GemmArgs& g, hipStream_t stream) {
   switch (tile) {
     case TILE_256x256_W8: return launch_routed_gemm<typename Tiles::T0>(g, stream);
-    case TILE_256x256_W4: return launch_routed_gemm<typename Tiles::T1>(g, stream);
+    case TILE_256x256_W4:
+      // The four-wave tile exists on the direct path only: staged through registers its 256 accumulators and the
+      // staging registers do not fit (the compiler spills some 430 of them); the eight-wave tile covers the same
+      // macro tile with half the accumulators per lane.
+      if constexpr (Tiles::T1::DIRECT) return launch_routed_gemm<typename Tiles::T1>(g, stream);
+      else return launch_routed_gemm<typename Tiles::T0>(g, stream);
     case TILE_128x128_W4: return launch_routed_gemm<typename Tiles::T2>(g, stream);
     case TILE_SMALL_W4: return launch_routed_gemm<typename Tiles::T3>(g, stream);
     case TILE_128x128_R4: return launch_routed_gemm<typename Tiles::T4>(g, stream);
