@@ -12,8 +12,8 @@
 namespace ffnk {
 
 constexpr int kRouteThreads = 256;
-constexpr int kRouteRowsPerThread = 16;
-constexpr int kRouteChunk = kRouteThreads * kRouteRowsPerThread;  // 4096 rows per block
+constexpr int kRouteRowsPerThread = 4;
+constexpr int kRouteChunk = kRouteThreads * kRouteRowsPerThread;  // 1024 rows per block: the launch is latency-bound, short chains per thread
 
 // 16-bit mask of the non-zero bytes of a 16-byte vector (bit j = byte j).
 __device__ __forceinline__ uint32_t nonzero_bytes16(uint4 v) {
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_kernel(const uint8_t* __r
                                                                int32_t* __restrict__ perm,
                                                                int32_t* __restrict__ counts) {
   __shared__ int s_red[2][kRouteThreads / kWave];
-  __shared__ int s_scan[kRouteThreads];
+  __shared__ int s_wave[kRouteThreads / kWave];
   const int t = threadIdx.x;
   const int64_t lo = (int64_t)blockIdx.x * kRouteChunk;  // first row of this block's chunk
 
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_kernel(const uint8_t* __r
     counts[1] = M - tot;
   }
 
-  // Phase 2: this thread owns rows [r0, r0 + 16) of the chunk.
+  // Phase 2: this thread owns kRouteRowsPerThread consecutive rows of the chunk, from r0.
   const int64_t r0 = lo + (int64_t)t * kRouteRowsPerThread;
   uint32_t bits = 0;
 #pragma unroll
@@ -85,16 +85,19 @@ __global__ __launch_bounds__(kRouteThreads) void route_kernel(const uint8_t* __r
     if (r0 + j < M && mask[r0 + j] != 0) bits |= 1u << j;
   }
   const int c = __popc(bits);
-  s_scan[t] = c;
-  __syncthreads();
-  // Inclusive Hillis-Steele scan over 256 per-thread counts.
-  for (int off = 1; off < kRouteThreads; off <<= 1) {
-    int add = (t >= off) ? s_scan[t - off] : 0;
-    __syncthreads();
-    s_scan[t] += add;
-    __syncthreads();
+  // Inclusive scan of the per-thread counts: inside each wave by shuffles, across the four waves through LDS.
+  int incl = c;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int up = __shfl_up(incl, off);
+    if ((t & (kWave - 1)) >= off) incl += up;
   }
-  int vb = bef + s_scan[t] - c;  // visual rows before r0
+  if ((t & (kWave - 1)) == kWave - 1) s_wave[t / kWave] = incl;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kRouteThreads / kWave; ++w)
+    if (w < t / kWave) incl += s_wave[w];
+  int vb = bef + incl - c;  // visual rows before r0
 #pragma unroll
   for (int j = 0; j < kRouteRowsPerThread; ++j) {
     const int64_t r = r0 + j;
