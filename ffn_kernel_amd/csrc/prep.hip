@@ -76,8 +76,9 @@ hipError_t launch_strided_copy2d(const uint16_t* src, int64_t sr, int64_t sc, ui
 // dst[c, pos] = src[perm[p], c] over padded routed positions pos in [0, pad64(nv) + pad64(nt));
 // padding positions are written as zero so that they add nothing to a contraction over pos.
 // blockIdx.z selects one of two (src, dst) pairs so that g and x are transposed in one launch.
-// 64 positions x 64 columns per block: 16-byte row reads, scalar transposing LDS writes, 16-byte
-// reads of the transposed tile, 16-byte stores (8 consecutive positions of one column).
+// 64 positions x 64 columns per block: 16-byte row reads (two positions per thread), transposing LDS writes of
+// one dword per pair of positions, 16-byte reads of the transposed tile, 16-byte stores (8 consecutive positions
+// of one column).
 struct GatherTransposeArgs {
   const uint16_t* src[2]; int64_t ld_src[2];
   uint16_t* dst[2]; int64_t ld_dst;
@@ -88,7 +89,10 @@ struct GatherTransposeArgs {
 };
 
 __global__ __launch_bounds__(256) void gather_transpose_kernel(const GatherTransposeArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t tile[kTt][kTt + 8];  // [column][position]
+  // [column][pair of positions], one dword per pair; the pair index is XORed with 4 * (column / 8 % 8), which keeps
+  // the transposing writes (a half wave: 8 column chunks x 4 pairs) and the 16-byte reads free of bank conflicts.
+  __shared__ __attribute__((aligned(16))) uint32_t tile[kTt][kTt / 2];
+  static_assert(kTt == 64, "one pass of 256 threads: 32 position pairs x 8 column chunks");
   const int z = blockIdx.z;
   const int cols = a.cols[z];
   const int c0 = blockIdx.y * kTt;
@@ -103,28 +107,30 @@ __global__ __launch_bounds__(256) void gather_transpose_kernel(const GatherTrans
   const uint16_t* src = a.src[z];
   const int64_t ld_src = a.ld_src[z];
   const int t = threadIdx.x;
-  const int ch = t & 7;  // 8-column chunk of the 64-column tile
+  const int ch = t & 7;   // 8-column chunk of the 64-column tile
+  const int pr = t >> 3;  // position pair inside the tile
+  const int c = c0 + ch * 8;
+  uint16_t v[2][8];
 #pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    const int i = (t >> 3) + pass * 32;  // position inside the tile
-    const int pos = pos0 + i;
+  for (int h = 0; h < 2; ++h) {
+    const int pos = pos0 + 2 * pr + h;
     const int p = text ? n_vis + (pos - vpad) : pos;
     const bool valid = text ? p < a.M : p < n_vis;
-    uint16_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    const int c = c0 + ch * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[h][e] = 0;
     if (valid) {
       const uint16_t* row = src + (int64_t)(a.routed[z] ? p : a.perm[p]) * ld_src;
       if (c + 8 <= cols) {
-        *reinterpret_cast<uint4*>(v) = *reinterpret_cast<const uint4*>(row + c);  // cols % 8 == 0, 16-byte aligned rows
+        *reinterpret_cast<uint4*>(v[h]) = *reinterpret_cast<const uint4*>(row + c);  // cols % 8 == 0, 16-byte aligned rows
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          if (c + e < cols) v[e] = row[c + e];
+          if (c + e < cols) v[h][e] = row[c + e];
       }
     }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) tile[ch * 8 + e][i] = v[e];
   }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) tile[ch * 8 + e][pr ^ (ch << 2)] = (uint32_t)v[0][e] | ((uint32_t)v[1][e] << 16);
   __syncthreads();
   uint16_t* dst = a.dst[z];
 #pragma unroll
@@ -132,7 +138,7 @@ __global__ __launch_bounds__(256) void gather_transpose_kernel(const GatherTrans
     const int cc = (t >> 3) + pass * 32;  // column inside the tile
     if (c0 + cc < cols)
       *reinterpret_cast<uint4*>(dst + (int64_t)(c0 + cc) * a.ld_dst + pos0 + ch * 8) =
-          *reinterpret_cast<const uint4*>(&tile[cc][ch * 8]);
+          *reinterpret_cast<const uint4*>(&tile[cc][(ch ^ ((cc >> 3) & 7)) << 2]);
   }
 }
 
