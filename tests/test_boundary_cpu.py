@@ -42,8 +42,14 @@ def test_tile_table_entries():
     big = _lib.tile_config(_lib.OP_FFN_UP, 32768, 4096, 14336)
     assert big["path"] == _lib.PATH_MFMA_TILED and big["block_m"] == 256 and big["direct_lds"] == 1
     assert big["block_k"] == 64 and big["lds_stages"] == 2  # two 64-element slabs, loaded global->LDS
+    assert big["waves_m"] * big["waves_n"] == 4  # four waves of 128x128
     half = _lib.tile_config(_lib.OP_LINEAR_FWD, 2048, 96, 1024)
     assert half["direct_lds"] == 0  # the direct path moves whole 128-byte lines: K % 64 == 0
+    # the four-wave 256x256 tile exists on the direct path only; a staged shape that would pick it runs eight waves
+    long_k = _lib.tile_config(_lib.OP_LINEAR_FWD, 32768, 4096, 4096)
+    assert long_k["direct_lds"] == 1 and long_k["block_m"] == 256 and long_k["waves_m"] * long_k["waves_n"] == 4
+    staged = _lib.tile_config(_lib.OP_LINEAR_FWD, 32768, 4096 + 8, 4096)
+    assert staged["direct_lds"] == 0 and staged["block_m"] == 256 and staged["waves_m"] * staged["waves_n"] == 8
     # M <= 8: dot-product streams, one wavefront per 1024-element K slice, no cross-workgroup split
     dec = _lib.tile_config(_lib.OP_FFN_FWD, 8, 4096, 14336)
     assert dec["path"] == _lib.PATH_STREAM and dec["lds_stages"] == 0 and dec["block_m"] == 8

@@ -766,7 +766,7 @@ def force_tile():
 
 
 @pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
-@pytest.mark.parametrize("M,K,N,p", [(700, 256, 512, 0.5), (333, 192, 320, 0.3), (1100, 1024, 264, 1.0)])
+@pytest.mark.parametrize("M,K,N,p", [(700, 256, 512, 0.5), (333, 192, 320, 0.3), (1100, 1024, 264, 1.0), (500, 200, 264, 0.5)])
 def test_forced_tile_linear_fwd_bwd(dev, force_tile, tile, M, K, N, p):
     """Each of the four tile shapes every GEMM family is compiled for (256x256 with 8 or 4 waves,
     128x128, 128x64, 128x128 behind a four-stage ring) runs the MaskedLinear forward and backward: the table alone never picks all of
