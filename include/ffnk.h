@@ -112,7 +112,7 @@ FFNK_API size_t ffnk_workspace_bytes_ffn_bwd(int64_t M, int64_t d, int64_t h, in
 FFNK_API int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t* out);
 
 /*
- * Tuner-only hooks (python -m ffn_kernel_amd.tune, the counterpart of the reference's find_spec/*.py
+ * Tuner-only hooks (python -m ffn_kernel_amd.tune, the counterpart of the reference's find_spec scripts
  * sweeps, and the tests that run every compiled tile).  ffnk_debug_force_tile: every LDS-tiled GEMM
  * launched by this process uses tile id `tile` (0 = 256x256 / 8 waves, 1 = 256x256 / 4 waves,
  * 2 = 128x128 / 4 waves, 3 = small, 4 = 128x128 / 4 waves behind a ring of four LDS stages); -1 returns to the tile table (measured plans first, then the
