@@ -44,8 +44,8 @@ GEN_PATH = Path(__file__).resolve().parent / "csrc" / "tile_table_gen.hpp"
 # M buckets [lo, hi]; each is measured at its upper end.  Below 65 rows the FFN runs the streaming kernels.
 BUCKETS = [(65, 128), (129, 256), (257, 512), (513, 1024), (1025, 2048), (2049, 4096), (4097, 8192), (8193, 16384),
            (16385, 32768)]
-FFN_LAYERS = [(1024, 2048), (2048, 8192), (4096, 14336)]    # (d, h): cfg2, a mid-size layer, cfg4 / cfg5
-LINEAR_LAYERS = [(1024, 1024), (2048, 2048), (4096, 4096)]  # (K, N): cfg1 / cfg3 and LLM-size projections
+FFN_LAYERS = [(1024, 2048), (2048, 8192), (4096, 14336), (5120, 13824), (8192, 28672)]  # (d, h): cfg2, a mid-size layer, cfg4 / cfg5, two larger LLM layers
+LINEAR_LAYERS = [(1024, 1024), (2048, 2048), (4096, 4096), (8192, 8192)]  # (K, N): cfg1 / cfg3 and LLM-size projections
 
 
 class _Events:
