@@ -3,6 +3,7 @@ MI355X (BASELINE.json's metric, `configs[3]`).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
                     [--workload cfg4|cfg2|cfg1|cfg3|decode1v|decode1t|decode8|decode32|decode64|decode64v|prefill1024]
+                    [--no-route-cache]
 
 A step is one pass of the hot path over the whole synthetic batch, inputs already resident in HBM:
   cfg4 / cfg2 / decodeN / prefillN : one MaskedFFN.apply (row partition + up-projection with SwiGLU +
@@ -232,7 +233,8 @@ def _bench_linear(args, dev) -> dict:
         "metric": metric, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic", "pct_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
-        "config": {"workload": w_cpu.name, "M": M, "K": K, "N": N, "visual_rows": int(w_cpu.mask.sum()), "tile": tile},
+        "config": {"workload": w_cpu.name, "M": M, "K": K, "N": N, "visual_rows": int(w_cpu.mask.sum()), "tile": tile,
+                   "row_partition": "per call" if args.no_route_cache else "shared between calls with the same mask"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": measured_traffic(args.workload),
                      "kernel": kernels, "kernel_ms": dev_avg, "kernel_ms_min": min(dev_ms), "algorithmic_flops": flops},
@@ -253,10 +255,14 @@ def main() -> int:
     ap.add_argument("--cpu-rows", type=int, default=1 << 30,
                     help="upper bound on the rows of the workload timed on the CPU (0 = skip); the sample is "
                          "sized to about 5 s per run")
+    ap.add_argument("--no-route-cache", action="store_true",
+                    help="partition the rows anew in every call instead of sharing one partition between calls "
+                         "that run with the same mask (ffn_kernel_amd.set_route_cache); a model's layers all "
+                         "route by one mask, so the default measures a call as a layer sees it")
     ap.add_argument("--no-decode", action="store_true",
                     help="cfg4 only: skip the decode-shape measurements (roofline_decode), e.g. under a profiler")
     args = ap.parse_args()
-    big = args.workload in ("cfg4", "gemm_ref", "copy1g")
+    big = args.workload in ("cfg4", "gemm_ref", "gemm_ref_down", "copy1g")
     if args.steps is None:
         args.steps = 20 if big else 200
     if args.warmup is None:
@@ -273,6 +279,9 @@ def main() -> int:
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.no_route_cache:
+        from ffn_kernel_amd import set_route_cache
+        set_route_cache(False)
     if args.workload == "copy1g":
         # Calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of exactly 1 GiB
         # (reads 1 GiB, writes 1 GiB per launch).  Not a benchmark of this library.
@@ -283,14 +292,16 @@ def main() -> int:
         torch.cuda.synchronize()
         print(json.dumps({"workload": "copy1g", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
         return 0
-    if args.workload == "gemm_ref":
-        # Reference point for the up-projection kernel: the vendor library's plain bf16 GEMM
-        # (torch's F.linear) on the shape the up-projection + SwiGLU launch computes at cfg4,
-        # [32768, 4096] x [28672, 4096]^T.  Not a benchmark of this library; run under rocprofv3
-        # to read the vendor kernel's launch geometry and counters beside routed_gemm_kernel's.
+    if args.workload in ("gemm_ref", "gemm_ref_down"):
+        # Reference points for the two GEMM launches of cfg4: the vendor library's plain bf16 GEMM
+        # (torch's F.linear) on the shape the up-projection + SwiGLU launch computes,
+        # [32768, 4096] x [28672, 4096]^T (gemm_ref), and on the down projection's,
+        # [32768, 14336] x [4096, 14336]^T (gemm_ref_down).  Not a benchmark of this library; run under
+        # rocprofv3 to read the vendor kernel's launch geometry and counters beside routed_gemm_kernel's.
+        gm, gn, gk = (32768, 28672, 4096) if args.workload == "gemm_ref" else (32768, 4096, 14336)
         g = torch.Generator().manual_seed(0)
-        a = torch.randn(32768, 4096, generator=g).to(torch.bfloat16).to(dev)
-        b = (torch.randn(28672, 4096, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+        a = torch.randn(gm, gk, generator=g).to(torch.bfloat16).to(dev)
+        b = (torch.randn(gn, gk, generator=g) * 0.02).to(torch.bfloat16).to(dev)
         for _ in range(args.warmup):
             torch.nn.functional.linear(a, b)
         torch.cuda.synchronize()
@@ -299,8 +310,8 @@ def main() -> int:
             torch.nn.functional.linear(a, b)
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        print(json.dumps({"workload": "gemm_ref", "M": 32768, "N": 28672, "K": 4096, "ms_per_step": ms,
-                          "tflops": 2 * 32768 * 28672 * 4096 / (ms * 1e-3) / 1e12}))
+        print(json.dumps({"workload": args.workload, "M": gm, "N": gn, "K": gk, "ms_per_step": ms,
+                          "tflops": 2 * gm * gn * gk / (ms * 1e-3) / 1e12}))
         return 0
     if args.workload in ("cfg1", "cfg3"):
         print(json.dumps(_bench_linear(args, dev)), flush=True)
@@ -398,7 +409,8 @@ def main() -> int:
         "data": "synthetic",
         "pct_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
         "config": {"workload": w_cpu.name, "M": M, "d": w.d, "h": w.h,
-                   "visual_rows": int(w_cpu.mask.sum()), "tile": tile},
+                   "visual_rows": int(w_cpu.mask.sum()), "tile": tile,
+                   "row_partition": "per call" if (args.no_route_cache or decode) else "shared between calls with the same mask"},
         "roofline": roofline,
     }
     if args.workload == "cfg4" and not args.no_decode:

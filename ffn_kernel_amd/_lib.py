@@ -48,6 +48,27 @@ _SIGNATURES = {
                                     c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,  # dW1 dW3 dU1 dU3
                                     c_void_p, c_void_p, c_int64, c_int64,            # dW2 dU2
                                     c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    # the *_routed variants: the plain signature (+ pre where optional) + const ffnk_routing_t*
+    "ffnk_masked_linear_fwd_routed": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p,
+                                              c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_size_t,
+                                              c_void_p, c_void_p]),
+    "ffnk_masked_linear_bwd_routed": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+                                              c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+                                              c_int64, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p,
+                                              c_void_p]),
+    "ffnk_masked_ffn_fwd_routed": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                           c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64,
+                                           c_void_p, c_int64,                        # pre (NULL: not kept)
+                                           c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p, c_void_p]),
+    "ffnk_masked_ffn_bwd_routed": (c_int, [c_void_p, c_int64, c_void_p, c_int64,
+                                           c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                           c_void_p, c_void_p, c_int64, c_int64,
+                                           c_void_p,
+                                           c_void_p, c_int64,                        # pre (NULL: recompute)
+                                           c_void_p, c_int64,
+                                           c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                           c_void_p, c_void_p, c_int64, c_int64,
+                                           c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p, c_void_p]),
     "ffnk_masked_ffn_can_save": (c_int, [c_int64, c_int64, c_int64]),
     "ffnk_masked_ffn_fwd_save": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                          c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64,
@@ -73,6 +94,11 @@ class TileConfig(ctypes.Structure):
 
     def as_dict(self) -> dict:
         return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+class RoutingStruct(ctypes.Structure):
+    """Mirror of ffnk_routing_t: device addresses of perm int32[M] and counts int32[2]."""
+    _fields_ = [("perm", c_void_p), ("counts", c_void_p)]
 
 
 class FfnkError(RuntimeError):

@@ -38,10 +38,11 @@ int hip_fail(hipError_t e, const char* what) {
     if (e__ != hipSuccess) return hip_fail(e__, what); \
   } while (0)
 
-// Row limit: the row partition runs in one launch whose blocks each re-count the mask bytes ahead of
-// their 4096-row chunk (M * M / 8192 bytes of L2 reads in total).  At 2^22 rows that is 2 GB, about
-// half a millisecond; beyond it the quadratic term would dominate the GEMMs it serves.
-constexpr int64_t kMaxRows = (int64_t)1 << 22;
+// Row limit.  The row partition runs in one launch of at most 256 blocks (route.hip), each of which
+// counts the whole mask once: 256 * M bytes of L2 / HBM reads, 4 GB and about a millisecond at 2^24 rows -
+// linear in M, and small against any GEMM over that many rows.  The tile counts and workspace offsets
+// derived from M stay inside 32-bit grids up to here for every N the column limit admits.
+constexpr int64_t kMaxRows = (int64_t)1 << 24;
 constexpr int64_t kMaxCols = (int64_t)1 << 24;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -84,6 +85,26 @@ int forced_splits() {
 }
 
 int64_t padded_rows(int64_t M) { return round_up64(M, 64) + 64; }  // >= pad64(nv) + pad64(M - nv)
+
+// The row partition a call works with: the caller's (ffnk_routing_t, made by ffnk_route for the same mask
+// and M) or, without one, the workspace's own region, filled by a route launch at the head of the call.
+struct Routing {
+  const int32_t* perm;
+  const int32_t* counts;
+};
+int resolve_routing(const ffnk_routing_t* rt, const RouteWs& r, const uint8_t* mask, int64_t M, hipStream_t stream,
+                    Routing* out) {
+  if (rt != nullptr) {
+    if (!rt->perm || !rt->counts) return fail(FFNK_E_NULL, "routing: perm or counts is NULL");
+    out->perm = rt->perm;
+    out->counts = rt->counts;
+    return FFNK_OK;
+  }
+  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+  out->perm = r.perm;
+  out->counts = r.counts;
+  return FFNK_OK;
+}
 
 struct BwdPlan {
   bool dw_k_contig;  // dW memory is [N, K] (k contiguous): R = N, Cc = K
@@ -191,15 +212,26 @@ static __device__ __align__(256) unsigned char scratch[FFNK_STATIC_SCRATCH_BYTES
 constexpr int kMaxDevices = 64;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
-// Address of `scratch` on the current device (looked up once per device; two threads that race
-// here both get the same answer).
-int static_scratch(void** out) {
-  int dev = -1;
-  FFNK_HIP(hipGetDevice(&dev), "hipGetDevice");
+// Address of `scratch` on the GPU that holds `on_device` (the call's output): each GPU has its own copy
+// of the array at its own address, and the kernels run where their operands live, which need not be the
+// calling thread's current device.  Looked up once per device, with that device current (two threads that
+// race here both get the same answer).
+int static_scratch(const void* on_device, void** out) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, on_device) != hipSuccess || attr.type != hipMemoryTypeDevice) {
+    (void)hipGetLastError();  // the query's own error must not surface in a later call
+    return fail(FFNK_E_NULL, "ffnk_masked_ffn_fwd_static: out is not device memory");
+  }
+  const int dev = attr.device;
   if (dev < 0 || dev >= kMaxDevices) return fail(FFNK_E_SHAPE, "device index %d outside [0, %d)", dev, kMaxDevices);
   void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if (p == nullptr) {
-    FFNK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    int cur = -1;
+    FFNK_HIP(hipGetDevice(&cur), "hipGetDevice");
+    if (cur != dev) FFNK_HIP(hipSetDevice(dev), "hipSetDevice");
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (cur != dev) FFNK_HIP(hipSetDevice(cur), "hipSetDevice");
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
     if (p == nullptr) return fail(FFNK_E_NULL, "static scratch has no address on device %d", dev);
     g_scratch_ptr[dev].store(p, std::memory_order_release);
   }
@@ -207,9 +239,9 @@ int static_scratch(void** out) {
   return FFNK_OK;
 }
 
-int routed_tile(int64_t M, int64_t n_out, bool dual, int64_t K = 0) {
+int routed_tile(int64_t M, int64_t n_out, bool dual, int64_t K = 0, int op = TUNED_PLAIN) {
   const int f = forced_tile();
-  return f >= 0 ? f : pick_routed_tile(M, n_out, dual, K, use_tuned());
+  return f >= 0 ? f : pick_routed_tile(M, n_out, dual, K, use_tuned(), op);
 }
 
 bool use_stream_path(int64_t M, int64_t d, int64_t h) { return stream_shape_ok(M, d, h); }
@@ -238,13 +270,14 @@ int down_splits(int64_t M, int64_t d, int64_t h) {
 // Split-K factor of the down projection on the LDS-tiled path (1: none).
 // Tile and split-K factor of the down projection on the LDS-tiled path (a forced tile keeps its own
 // best split).
-RoutedPlan down_plan(int64_t M, int64_t d, int64_t h) {
+// `op`: whose measured plans apply (TunedOp).
+RoutedPlan down_plan(int64_t M, int64_t d, int64_t h, int op = TUNED_DOWN) {
   RoutedPlan p;
   if (const int f = forced_tile(); f >= 0) {
     p.tile = f;
     p.splits = pick_routed_splits(M, d, h, p.tile);
   } else {
-    p = pick_routed_plan(M, d, h, use_tuned());
+    p = pick_routed_plan(M, d, h, use_tuned(), op);
   }
   // a forced split-K factor: whole 64-element slabs, no empty range, what the reduce pass can address
   if (const int fs = forced_splits(); fs >= 1 && h % 64 == 0 && M < 65536 && cdiv64(h / 64, cdiv64(h / 64, fs)) == fs &&
@@ -255,10 +288,12 @@ RoutedPlan down_plan(int64_t M, int64_t d, int64_t h) {
 // dx GEMM of the MaskedFFN backward: few output tiles over a 2h-long contraction, so K is split like the forward's
 // down projection when the fp32 partials fit `room`; an unsplit big tile wants room for its split tail instead.
 RoutedPlan ffn_bwd_dx_plan(int64_t M, int64_t d, int64_t h, bool dx_direct, size_t room, size_t* need) {
-  RoutedPlan dxp = down_plan(M, d, 2 * h);
+  // Rules and cost model only: the measured plans are timings of other kernels (the forward's down
+  // projection reads K-contiguous weights through another loop).
+  RoutedPlan dxp = down_plan(M, d, 2 * h, TUNED_NONE);
   if (!dx_direct || (size_t)dxp.splits * M * d * 4 > room) {
     dxp.splits = 1;
-    dxp.tile = routed_tile(M, d, false);
+    dxp.tile = routed_tile(M, d, false, 0, TUNED_NONE);
   }
   size_t n = 0;
   if (dxp.splits > 1) n = (size_t)dxp.splits * M * d * 4;
@@ -307,9 +342,9 @@ int linear_stream_splits(int64_t M, int64_t K, int64_t N) {
 
 // MaskedLinear forward: the table's tile unless cutting K pays (few output tiles, long contraction).
 RoutedPlan linear_plan(int64_t M, int64_t K, int64_t N) {
-  RoutedPlan p = down_plan(M, N, K);
+  RoutedPlan p = down_plan(M, N, K, TUNED_PLAIN);
   if (N % 4 != 0) p.splits = 1;  // the reduce pass moves four columns per thread
-  if (p.splits == 1) p.tile = routed_tile(M, N, false, K);
+  if (p.splits == 1) p.tile = routed_tile(M, N, false, K, TUNED_PLAIN);
   return p;
 }
 // fp32 partials of the tiled MaskedLinear forward: split-K for the whole GEMM, or the split tail of
@@ -340,7 +375,6 @@ size_t tiled_down_partial_bytes(int64_t M, int64_t d, int64_t h) {
 // contraction shortens the estimate by more than 40 % (at M = 8192, K = N = 1024 two ranges measure 7 % slower than one); never more ranges than the plan sized
 // the partials for.
 int fused_bwd_splits(int64_t M, int64_t K, int64_t N, int plan_splits) {
-  if (forced_splits() >= 1) return plan_splits;  // the tuner's factor went into the plan
   const double slots = 2.0 * kCus, t_slab = 0.8;
   const double dw_tiles = 2.0 * (double)cdiv64(N, 128) * (double)cdiv64(K, 128);
   const double dx_units = (double)(cdiv64(M, 128) + 1) * (double)cdiv64(K, 128) * (double)cdiv64(N, 64);
@@ -362,6 +396,17 @@ int fused_bwd_splits(int64_t M, int64_t K, int64_t N, int plan_splits) {
     }
   }
   return best_t < 0.6 * unsplit ? best : 1;
+}
+
+// Whether the MaskedLinear backward runs its two GEMMs in one launch, and the split-K factor its
+// weight-gradient GEMM is really launched with.  A measured plan and a forced factor are used as they are
+// (that is what the tuner timed); only a factor the rules guessed goes through the fused launch's own model.
+bool bwd_is_fused(int64_t M, int64_t K, const BwdPlan& p, bool w_kmajor) {
+  return w_kmajor && routed_tile(M, K, false, 0, TUNED_NONE) == TILE_128x128_W4 && p.tc.tile == TILE_128x128_W4;
+}
+int bwd_dw_launch_splits(int64_t M, int64_t K, int64_t N, const BwdPlan& p, bool fused) {
+  if (!fused || p.tc.tuned || forced_splits() >= 1) return p.tc.splits;
+  return fused_bwd_splits(M, K, N, p.tc.splits);
 }
 
 }  // namespace
@@ -441,10 +486,14 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
     case FFNK_OP_FFN_UP: tile = routed_tile(M, N, true, K); dual = true; contraction = K; break;
     case FFNK_OP_FFN_DOWN: tile = down_plan(M, K, N).tile; contraction = N; break;  // out cols = d = K, contraction h = N
     case FFNK_OP_LINEAR_BWD:
-    case FFNK_OP_BWD_DX: tile = routed_tile(M, K, false); contraction = N; break;
+    case FFNK_OP_BWD_DX: tile = routed_tile(M, K, false, 0, TUNED_NONE); contraction = N; break;
     case FFNK_OP_BWD_DW: {
-      const TileChoice c = plan_bwd(M, K, N, true).tc;
-      tile = c.tile; splits = c.splits; contraction = M; break;
+      // As launched for the reference's layout (nn.Linear.weight.T views, contiguous g): weights read in place.
+      const BwdPlan bp = plan_bwd(M, K, N, true);
+      const bool w_kmajor = N > 0 && N % 64 == 0 && K >= 8 && K % 8 == 0 && direct_ok(N, M, N, 8);
+      tile = bp.tc.tile; contraction = M;
+      splits = bwd_dw_launch_splits(M, K, N, bp, bwd_is_fused(M, K, bp, w_kmajor));
+      break;
     }
     default: return fail(FFNK_E_OP, "unknown op %d", op);
   }
@@ -522,6 +571,14 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
                            int64_t w_stride_k, int64_t w_stride_n, const uint8_t* mask, uint16_t* y,
                            int64_t y_stride_m, int64_t M, int64_t K, int64_t N, void* ws, size_t ws_bytes,
                            void* stream_) {
+  return ffnk_masked_linear_fwd_routed(x, x_stride_m, Wv, Wt, w_stride_k, w_stride_n, mask, y, y_stride_m, M, K, N, ws,
+                                       ws_bytes, stream_, nullptr);
+}
+
+int ffnk_masked_linear_fwd_routed(const uint16_t* x, int64_t x_stride_m, const uint16_t* Wv, const uint16_t* Wt,
+                                  int64_t w_stride_k, int64_t w_stride_n, const uint8_t* mask, uint16_t* y,
+                                  int64_t y_stride_m, int64_t M, int64_t K, int64_t N, void* ws, size_t ws_bytes,
+                                  void* stream_, const ffnk_routing_t* routing) {
   hipStream_t stream = (hipStream_t)stream_;
   if (int e = check_extents(M, K, N)) return e;
   if (M == 0 || N == 0) return FFNK_OK;
@@ -564,12 +621,13 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
       FFNK_HIP(launch_stream_reduce(a.P, splits, (int)M, (int)N, mask, y, y_stride_m, stream), "streaming reduce");
     return FFNK_OK;
   }
-  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+  Routing rt;
+  if (int e = resolve_routing(routing, r, mask, M, stream, &rt)) return e;
   GemmArgs g;
   g.A = x; g.lda = x_stride_m;
   g.B0[0] = Wv; g.B0[1] = Wt; g.B1[0] = g.B1[1] = nullptr; g.ldb = w_stride_n;
   g.C = y; g.ldc = y_stride_m;
-  g.perm = r.perm; g.counts = r.counts;
+  g.perm = rt.perm; g.counts = rt.counts;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   const bool direct = direct_ok(K, M, x_stride_m, w_stride_n);
   RoutedPlan plan = linear_plan(M, K, N);
@@ -585,7 +643,7 @@ int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m, const uint16_t
   }
   FFNK_HIP(launch_linear_gemm(plan.tile, direct, g, stream), "linear GEMM");
   if (plan.splits > 1)
-    FFNK_HIP(launch_routed_reduce(g.P, plan.splits, (int)M, (int)N, r.perm, y, y_stride_m, stream), "linear reduce");
+    FFNK_HIP(launch_routed_reduce(g.P, plan.splits, (int)M, (int)N, rt.perm, y, y_stride_m, stream), "linear reduce");
   return FFNK_OK;
 }
 
@@ -608,7 +666,7 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
                  const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n, const uint16_t* W2, const uint16_t* U2,
                  int64_t down_stride_k, int64_t down_stride_n, const uint8_t* mask, uint16_t* out, int64_t out_stride_m,
                  uint16_t* pre, int64_t pre_stride_m, int64_t M, int64_t d, int64_t h, void* ws, size_t ws_bytes,
-                 void* stream_, void* const* events) {
+                 void* stream_, void* const* events, const ffnk_routing_t* routing = nullptr) {
   hipStream_t stream = (hipStream_t)stream_;
   auto mark = [&](int i) -> hipError_t {
     if (events && events[i]) return hipEventRecord((hipEvent_t)events[i], stream);
@@ -695,13 +753,14 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
     return FFNK_OK;
   }
 
-  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+  Routing rt;
+  if (int e = resolve_routing(routing, r, mask, M, stream, &rt)) return e;
   FFNK_HIP(mark(0), "event record");
   GemmArgs up;
   up.A = x; up.lda = x_stride_m;
   up.B0[0] = W1; up.B0[1] = U1; up.B1[0] = W3; up.B1[1] = U3; up.ldb = up_stride_n;
   up.C = H; up.ldc = ldh;
-  up.perm = r.perm; up.counts = r.counts;
+  up.perm = rt.perm; up.counts = rt.counts;
   up.M = (int)M; up.N = (int)h; up.K = (int)d;
   up.C_pre = pre; up.ldc_pre = pre_stride_m;
   FFNK_HIP(launch_up_gemm(routed_tile(M, h, true, d), direct_ok(d, M, x_stride_m, up_stride_n), up, stream), "up-projection GEMM");
@@ -710,7 +769,7 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
   dn.A = H; dn.lda = ldh;
   dn.B0[0] = W2; dn.B0[1] = U2; dn.B1[0] = dn.B1[1] = nullptr; dn.ldb = down_stride_n;
   dn.C = out; dn.ldc = out_stride_m;
-  dn.perm = r.perm; dn.counts = r.counts;
+  dn.perm = rt.perm; dn.counts = rt.counts;
   dn.M = (int)M; dn.N = (int)d; dn.K = (int)h;
   const bool dn_direct = direct_ok(h, 0, ldh, down_stride_n);
   const int dn_splits = dn_direct ? tiled_down_splits(M, d, h) : 1;
@@ -723,7 +782,7 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
   }
   FFNK_HIP(launch_down_gemm(down_tile(M, d, h), dn_direct, dn, stream), "down-projection GEMM");
   if (dn_splits > 1)
-    FFNK_HIP(launch_routed_reduce(dn.P, dn_splits, (int)M, (int)d, r.perm, out, out_stride_m, stream), "down-projection reduce");
+    FFNK_HIP(launch_routed_reduce(dn.P, dn_splits, (int)M, (int)d, rt.perm, out, out_stride_m, stream), "down-projection reduce");
   FFNK_HIP(mark(2), "event record");
   return FFNK_OK;
 }
@@ -752,12 +811,24 @@ int ffnk_masked_ffn_fwd_static(const uint16_t* x, int64_t x_stride_m, const uint
     return fail(FFNK_E_WORKSPACE, "ffnk_masked_ffn_fwd_static: M=%lld d=%lld h=%lld needs %zu bytes of scratch, the static "
                                   "buffer holds %zu; use ffnk_masked_ffn_fwd with a workspace",
                 (long long)M, (long long)d, (long long)h, need, (size_t)FFNK_STATIC_SCRATCH_BYTES);
+  if (M == 0 || d == 0) return FFNK_OK;
+  if (!out) return fail(FFNK_E_NULL, "x, mask or out is NULL");
   void* ws = nullptr;
-  if (int e = static_scratch(&ws)) return e;
+  if (int e = static_scratch(out, &ws)) return e;
   // Nothing in the scratch has to start at zero: every region the forward reads (perm, counts, the
   // intermediate, the fp32 partials) is written by an earlier kernel of the same call.
   return ffn_fwd_impl(x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k, down_stride_n, mask,
                       out, out_stride_m, nullptr, 0, M, d, h, ws, (size_t)FFNK_STATIC_SCRATCH_BYTES, stream_, nullptr);
+}
+
+int ffnk_masked_ffn_fwd_routed(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, const uint16_t* W3,
+                               const uint16_t* U1, const uint16_t* U3, int64_t up_stride_k, int64_t up_stride_n,
+                               const uint16_t* W2, const uint16_t* U2, int64_t down_stride_k, int64_t down_stride_n,
+                               const uint8_t* mask, uint16_t* out, int64_t out_stride_m, uint16_t* pre,
+                               int64_t pre_stride_m, int64_t M, int64_t d, int64_t h, void* ws, size_t ws_bytes,
+                               void* stream_, const ffnk_routing_t* routing) {
+  return ffn_fwd_impl(x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k, down_stride_n, mask,
+                      out, out_stride_m, pre, pre_stride_m, M, d, h, ws, ws_bytes, stream_, nullptr, routing);
 }
 
 int ffnk_masked_ffn_can_save(int64_t M, int64_t d, int64_t h) {
@@ -780,6 +851,15 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
                            const uint8_t* mask, uint16_t* dx, int64_t dx_stride_m, uint16_t* dWv, uint16_t* dWt,
                            int64_t dw_stride_k, int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, void* ws,
                            size_t ws_bytes, void* stream_) {
+  return ffnk_masked_linear_bwd_routed(g, g_stride_m, x, x_stride_m, Wv, Wt, w_stride_k, w_stride_n, mask, dx, dx_stride_m,
+                                       dWv, dWt, dw_stride_k, dw_stride_n, M, K, N, ws, ws_bytes, stream_, nullptr);
+}
+
+int ffnk_masked_linear_bwd_routed(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,
+                                  const uint16_t* Wv, const uint16_t* Wt, int64_t w_stride_k, int64_t w_stride_n,
+                                  const uint8_t* mask, uint16_t* dx, int64_t dx_stride_m, uint16_t* dWv, uint16_t* dWt,
+                                  int64_t dw_stride_k, int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, void* ws,
+                                  size_t ws_bytes, void* stream_, const ffnk_routing_t* routing) {
   hipStream_t stream = (hipStream_t)stream_;
   if (int e = check_extents(M, K, N)) return e;
   if (K == 0) return FFNK_OK;  // dx and dW are empty
@@ -809,7 +889,8 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   if (!aligned16(ws)) return fail(FFNK_E_ALIGN, "workspace not 16-byte aligned");
   uint8_t* wsb = static_cast<uint8_t*>(ws);
   const RouteWs r = carve_route(wsb, M);
-  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+  Routing rt;
+  if (int e = resolve_routing(routing, r, mask, M, stream, &rt)) return e;
 
   // ---- dx = gather(g) @ W_g^T, contraction over N: needs the weights as [K, N] rows, N contiguous ----
   const uint16_t* wt[2] = {Wv, Wt};
@@ -830,12 +911,12 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   a.A = g; a.lda = g_stride_m;
   a.B0[0] = wt[0]; a.B0[1] = wt[1]; a.B1[0] = a.B1[1] = nullptr; a.ldb = ldw;
   a.C = dx; a.ldc = dx_stride_m;
-  a.perm = r.perm; a.counts = r.counts;
+  a.perm = rt.perm; a.counts = rt.counts;
   a.M = (int)M; a.N = (int)K; a.K = (int)N;
-  const int dx_tile = routed_tile(M, K, false);
+  const int dx_tile = routed_tile(M, K, false, 0, TUNED_NONE);
   // Both GEMMs on the 128x128 tile and the weights readable in place: one launch runs the two side by
   // side (after the transposes it depends on), see below.
-  const bool fused = w_kmajor && dx_tile == TILE_128x128_W4 && p.tc.tile == TILE_128x128_W4;
+  const bool fused = bwd_is_fused(M, K, p, w_kmajor);
   if (!fused) {
     if (w_kmajor) FFNK_HIP(launch_linear_gemm_kmajor(dx_tile, a, stream), "dx GEMM");
     else FFNK_HIP(launch_linear_gemm(dx_tile, direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
@@ -845,16 +926,16 @@ int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t
   uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]
   uint16_t* XT = reinterpret_cast<uint16_t*>(wsb + p.off_xt);  // [K, ldt]
   float* P = reinterpret_cast<float*>(wsb + p.off_p);
-  FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)N, GT, x, x_stride_m, (int)K, XT, p.ldt, r.perm, r.counts,
+  FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)N, GT, x, x_stride_m, (int)K, XT, p.ldt, rt.perm, rt.counts,
                                     (int)M, stream), "g / x transpose");
   SplitKArgs s;
   s.A = p.dw_k_contig ? GT : XT; s.lda = p.ldt;
   s.B = p.dw_k_contig ? XT : GT; s.ldb = p.ldt;
-  s.P = P; s.counts = r.counts; s.M = (int)M;
+  s.P = P; s.counts = rt.counts; s.M = (int)M;
   s.R = (int)p.R; s.Cc = (int)p.Cc; s.splits = p.tc.splits;
   const int64_t sr = p.dw_k_contig ? dw_stride_n : dw_stride_k;
   const int64_t sc = p.dw_k_contig ? dw_stride_k : dw_stride_n;
-  if (fused) s.splits = fused_bwd_splits(M, K, N, p.tc.splits);
+  s.splits = bwd_dw_launch_splits(M, K, N, p, fused);
   if (s.splits == 1) { s.out[0] = dWv; s.out[1] = dWt; s.out_sr = sr; s.out_sc = sc; }
   if (fused) FFNK_HIP(launch_fused_bwd(a, s, stream), "fused dx / dW GEMM");
   else FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
@@ -875,7 +956,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
                  const uint8_t* mask, const uint16_t* pre, int64_t pre_stride_m, uint16_t* dx, int64_t dx_stride_m,
                  uint16_t* dW1, uint16_t* dW3, uint16_t* dU1, uint16_t* dU3, int64_t dup_stride_k, int64_t dup_stride_n,
                  uint16_t* dW2, uint16_t* dU2, int64_t ddown_stride_k, int64_t ddown_stride_n, int64_t M, int64_t d,
-                 int64_t h, void* ws, size_t ws_bytes, void* stream_) {
+                 int64_t h, void* ws, size_t ws_bytes, void* stream_, const ffnk_routing_t* routing = nullptr) {
   hipStream_t stream = (hipStream_t)stream_;
   if (pre != nullptr && (pre_stride_m < 2 * h || pre_stride_m % 8 != 0 || !aligned16(pre)))
     return fail(FFNK_E_STRIDE, "pre_stride_m=%lld: need >= 2h, a multiple of 8, and 16-byte aligned rows",
@@ -909,13 +990,14 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   const RouteWs r = carve_route(wsb, M);
   uint16_t* T13 = reinterpret_cast<uint16_t*>(wsb + p.off_t13);
   uint16_t* DH = reinterpret_cast<uint16_t*>(wsb + p.off_dh);
-  FFNK_HIP(launch_route(mask, (int)M, r.perm, r.counts, stream), "route kernel");
+  Routing rt;
+  if (int e = resolve_routing(routing, r, mask, M, stream, &rt)) return e;
 
   // ---- pre-activations, routed order: T13[:, 0:h] = x A1, T13[:, h:2h] = x A3 ----
   GemmArgs a;
   a.A = x; a.lda = x_stride_m;
   a.B1[0] = a.B1[1] = nullptr; a.ldb = up_stride_n;
-  a.ldc = ld13; a.perm = r.perm; a.counts = r.counts;
+  a.ldc = ld13; a.perm = rt.perm; a.counts = rt.counts;
   a.M = (int)M; a.N = (int)h; a.K = (int)d;
   const bool up_direct = direct_ok(d, M, x_stride_m, up_stride_n);
   if (pre == nullptr) {
@@ -962,7 +1044,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
     FFNK_HIP(launch_strided_copy2d(U3, up_stride_k, up_stride_n, w13[1] + h, ld13, (int)d, (int)h, stream), "weight transpose");
     b.B0[0] = w13[0]; b.B0[1] = w13[1]; b.B1[0] = b.B1[1] = nullptr; b.ldb = ld13;
   }
-  b.C = dx; b.ldc = dx_stride_m; b.perm = r.perm; b.counts = r.counts;
+  b.C = dx; b.ldc = dx_stride_m; b.perm = rt.perm; b.counts = rt.counts;
   b.M = (int)M; b.N = (int)d; b.K = (int)(2 * h);
   // Few output tiles over a 2h-long contraction: split K like the forward's down projection.  The
   // fp32 partials live where the W2^T copies were (dead since the dh GEMM), if they fit there.
@@ -979,7 +1061,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   if (w13_kmajor) FFNK_HIP(launch_down_gemm_kmajor(dxp.tile, b, stream), "dx GEMM");
   else FFNK_HIP(launch_down_gemm(dxp.tile, dx_direct, b, stream), "dx GEMM");
   if (dxp.splits > 1)
-    FFNK_HIP(launch_routed_reduce(b.P, dxp.splits, (int)M, (int)d, r.perm, dx, dx_stride_m, stream), "dx reduce");
+    FFNK_HIP(launch_routed_reduce(b.P, dxp.splits, (int)M, (int)d, rt.perm, dx, dx_stride_m, stream), "dx reduce");
 
   // ---- weight gradients: contraction over the rows of each group.  x and g are gathered into
   // 64-padded transposes; H, dt1 and dt3 (routed order already) are read in place by the K-major
@@ -989,7 +1071,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   float* P = reinterpret_cast<float*>(wsb + p.off_p);
   const bool in_place = paths.acts_in_place;
   if (in_place) {
-    FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, x, x_stride_m, (int)d, XT, p.ldt, r.perm, r.counts, (int)M,
+    FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, x, x_stride_m, (int)d, XT, p.ldt, rt.perm, rt.counts, (int)M,
                                       stream, false, false), "g / x transpose");
     const TileChoice tc = ffn_bwd_in_place_choice(M, d, h);
     const int tile = forced_tile() >= 0 ? forced_tile() : tc.tile;
@@ -999,7 +1081,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
       SplitKArgs s;
       s.A = rows; s.lda = ld_rows;
       s.B = cT; s.ldb = p.ldt;
-      s.P = P; s.counts = r.counts; s.M = (int)M;
+      s.P = P; s.counts = rt.counts; s.M = (int)M;
       s.R = (int)h; s.Cc = (int)d; s.splits = tc.splits;
       if (tc.splits == 1) { s.out[0] = o0; s.out[1] = o1; s.out_sr = sr; s.out_sc = sc; }
       FFNK_HIP(launch_splitk_gemm_kmajor(tile, s, stream), "dW split-K GEMM");
@@ -1015,18 +1097,18 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   uint16_t* HT = reinterpret_cast<uint16_t*>(wsb + p.off_ht);    // [h, ldt]
   uint16_t* D1T = reinterpret_cast<uint16_t*>(wsb + p.off_d1t);  // [h, ldt]
   uint16_t* D3T = reinterpret_cast<uint16_t*>(wsb + p.off_d3t);  // [h, ldt]
-  FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, DH, h, (int)h, HT, p.ldt, r.perm, r.counts, (int)M,
+  FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)d, GT, DH, h, (int)h, HT, p.ldt, rt.perm, rt.counts, (int)M,
                                     stream, false, true), "g / intermediate transpose");
-  FFNK_HIP(launch_gather_transpose2(x, x_stride_m, (int)d, XT, T13, ld13, (int)h, D1T, p.ldt, r.perm, r.counts,
+  FFNK_HIP(launch_gather_transpose2(x, x_stride_m, (int)d, XT, T13, ld13, (int)h, D1T, p.ldt, rt.perm, rt.counts,
                                     (int)M, stream, false, true), "x / dt1 transpose");
-  FFNK_HIP(launch_gather_transpose2(T13 + h, ld13, (int)h, D3T, nullptr, 0, 0, nullptr, p.ldt, r.perm, r.counts,
+  FFNK_HIP(launch_gather_transpose2(T13 + h, ld13, (int)h, D3T, nullptr, 0, 0, nullptr, p.ldt, rt.perm, rt.counts,
                                     (int)M, stream, true, false), "dt3 transpose");
   auto weight_grad = [&](const BwdPlan& q, const uint16_t* gT, const uint16_t* xT, uint16_t* o0, uint16_t* o1,
                          int64_t sk, int64_t sn) -> int {
     SplitKArgs s;
     s.A = q.dw_k_contig ? gT : xT; s.lda = p.ldt;
     s.B = q.dw_k_contig ? xT : gT; s.ldb = p.ldt;
-    s.P = P; s.counts = r.counts; s.M = (int)M;
+    s.P = P; s.counts = rt.counts; s.M = (int)M;
     s.R = (int)q.R; s.Cc = (int)q.Cc; s.splits = q.tc.splits;
     const int64_t sr = q.dw_k_contig ? sn : sk, sc = q.dw_k_contig ? sk : sn;
     if (q.tc.splits == 1) { s.out[0] = o0; s.out[1] = o1; s.out_sr = sr; s.out_sc = sc; }
@@ -1056,6 +1138,19 @@ int ffnk_masked_ffn_bwd(const uint16_t* g, int64_t g_stride_m, const uint16_t* x
   return ffn_bwd_impl(g, g_stride_m, x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k,
                       down_stride_n, mask, nullptr, 0, dx, dx_stride_m, dW1, dW3, dU1, dU3, dup_stride_k, dup_stride_n,
                       dW2, dU2, ddown_stride_k, ddown_stride_n, M, d, h, ws, ws_bytes, stream_);
+}
+
+int ffnk_masked_ffn_bwd_routed(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,
+                               const uint16_t* W1, const uint16_t* W3, const uint16_t* U1, const uint16_t* U3,
+                               int64_t up_stride_k, int64_t up_stride_n, const uint16_t* W2, const uint16_t* U2,
+                               int64_t down_stride_k, int64_t down_stride_n, const uint8_t* mask, const uint16_t* pre,
+                               int64_t pre_stride_m, uint16_t* dx, int64_t dx_stride_m, uint16_t* dW1, uint16_t* dW3,
+                               uint16_t* dU1, uint16_t* dU3, int64_t dup_stride_k, int64_t dup_stride_n, uint16_t* dW2,
+                               uint16_t* dU2, int64_t ddown_stride_k, int64_t ddown_stride_n, int64_t M, int64_t d,
+                               int64_t h, void* ws, size_t ws_bytes, void* stream_, const ffnk_routing_t* routing) {
+  return ffn_bwd_impl(g, g_stride_m, x, x_stride_m, W1, W3, U1, U3, up_stride_k, up_stride_n, W2, U2, down_stride_k,
+                      down_stride_n, mask, pre, pre_stride_m, dx, dx_stride_m, dW1, dW3, dU1, dU3, dup_stride_k,
+                      dup_stride_n, dW2, dU2, ddown_stride_k, ddown_stride_n, M, d, h, ws, ws_bytes, stream_, routing);
 }
 
 int ffnk_masked_ffn_bwd_saved(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64_t x_stride_m,

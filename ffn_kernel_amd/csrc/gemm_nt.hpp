@@ -8,7 +8,8 @@
 // Data path per workgroup: 64-column K slabs of the A and B panels go global -> LDS, two stages
 // deep (directly, bypassing registers, when K is a multiple of 64; staged through registers
 // otherwise); wavefronts read 16-byte MFMA fragments from an XOR-swizzled LDS layout and issue
-// v_mfma_f32_32x32x16_bf16.
+// v_mfma_f32_16x16x32_bf16 on the 256-row direct tiles (gemm_mainloop_fixed16) and v_mfma_f32_32x32x16_bf16
+// on the others (gemm_mainloop_slab_dma, gemm_mainloop_ring, gemm_mainloop_staged).
 //
 // The backward GEMMs find one operand with the contraction running over its rows ([K, N], N
 // contiguous: a forward weight seen from the output side, or activations whose rows are summed).
@@ -106,8 +107,6 @@ struct RoutedGemmCfg {
   static constexpr bool B_KMAJOR = B_KMAJOR_;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int NT = NWAVES * kWave;
-  // One wavefront per SIMD: the K loop is a fixed, source-order schedule (see gemm_mainloop_slab_dma).
-  static constexpr bool FIXED_SCHEDULE = DIRECT_ && !B_KMAJOR_ && BM_ == 256;  // (32x32x16 form; superseded where MFMA16)
   static constexpr int BN_OUT = DUAL ? BN / 2 : BN;        // output columns per tile
   static constexpr int WTM = BM / WAVES_M;                 // rows per wave
   static constexpr int WTN_OUT = BN_OUT / WAVES_N;         // output columns per wave
@@ -530,83 +529,16 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
     kmajor_step(1, u ^ 1, s0, full || kt + 1 < nk, full || kt + 2 < nk, u, kt + 2);
   };
 
-  // ---- One wavefront per SIMD (four-wave tiles): no second wave fills a wait, and an instruction that
-  // cannot issue (a load while the address unit's queue is full) holds back the MFMAs behind it.  So the
-  // same pipeline is written out in source order, every MFMA fenced by scheduling barriers:
-  //  * the LDS reads of the next K step go one behind each of the first MFMAs of a step, a half step
-  //    ahead of their first use; the step before the barrier therefore finds them returned there;
-  //  * the global->LDS loads go out at the rate the address unit takes them (a 1 KB load per wave every
-  //    second MFMA, i.e. one per 16 cycles and CU) instead of in a burst behind the barrier: the first
-  //    half of the slab after next during the last K step of a slab, the second half during the first
-  //    K step of the following slab - still three quarters of a slab ahead of the barrier that needs them.
-  constexpr int FH = (L + 1) / 2;                         // loads per half
-  constexpr int FEV = NM / FH >= 1 ? NM / FH : 1;         // one load behind every FEV-th MFMA
-  static_assert(!Cfg::FIXED_SCHEDULE || (ND <= NM && FH <= NM), "fixed schedule: reads and loads must fit a K step");
-  auto fixed_reads = [&](int buf, int stage, auto step, int r) {
-    constexpr int ks = decltype(step)::value;
-    const uint8_t* st = lds + stage * STAGE;
-    if (r < TN) fb[buf][r] = *reinterpret_cast<const bf16x8_t*>(st + b_base[r] + koff[ks]);
-    else fa[buf][r - TN] = *reinterpret_cast<const bf16x8_t*>(st + a_base + (r - TN) * 32 * kRowBytes + koff[ks]);
-  };
-  // Load l of a slab: the weight panel's first (as at the head of the tile), then the token panel's.
-  auto fixed_load = [&](int l, int stage, int kt) {
-    uint8_t* st = lds + stage * STAGE;
-    const int ko = kt * kRowBytes;
-    if (l < NJB)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
-    else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l - NJB], FFNK_LDS_PTR(st + ((l - NJB) * NWAVES + wave) * 1024), 16,
-                                               offA[l - NJB], ko, 0, Cfg::AUX_A);
-  };
-  // One K step: MFMAs on fragment buffer `cur`; behind them the reads of (stage_next, step_next) into the
-  // other buffer and loads [l0, l0 + FH) of slab kt_dma into stage_dma.
-  auto fixed_step = [&](int cur, int stage_next, auto step_next, bool reads, bool dma, int l0, int stage_dma, int kt_dma) {
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int q = 0; q < NM; ++q) {
-      acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][q % TN], fa[cur][q / TN], acc[q / TN][q % TN], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (q < ND && reads) fixed_reads(cur ^ 1, stage_next, step_next, q);
-      if (q % FEV == FEV - 1 && q / FEV < FH && l0 + q / FEV < L && dma) fixed_load(l0 + q / FEV, stage_dma, kt_dma);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-  constexpr std::integral_constant<int, 0> f0{};
-  constexpr std::integral_constant<int, 1> f1{};
-  constexpr std::integral_constant<int, 2> f2{};
-  constexpr std::integral_constant<int, 3> f3{};
-  // Stage u holds slab kt.  On entry slab kt + 1 is half issued (its first FH loads) into the other stage.
-  auto fixed_body = [&](int u, int kt, bool full) {
-    fixed_step(0, u, f1, true, full || kt + 1 < nk, FH, u ^ 1, kt + 1);
-    fixed_step(1, u, f2, true, false, 0, 0, 0);
-    fixed_step(0, u, f3, true, false, 0, 0, 0);
-    dma_wait_barrier<0>();  // every wave has read the last of stage u; the next slab has landed in the other stage
-    fixed_step(1, u ^ 1, f0, full || kt + 1 < nk, full || kt + 2 < nk, 0, u, kt + 2);
-  };
-
   // Head of the tile: the weight panels of the first two slabs go out first - their addresses do not
   // depend on the routing - so that they fly while the gathered token rows' indices are still loading.
-  if constexpr (Cfg::FIXED_SCHEDULE) {
-    // slab 0 whole, slab 1's first half: the fixed schedule issues second halves during a slab's first K step
-    issue_b(0, 0);
-    issue_a(0, 0);
-    if (nk > 1) {
-#pragma unroll
-      for (int l = 0; l < FH; ++l) fixed_load(l, 1, 1);
-      dma_wait_barrier<FH>();
-    } else {
-      dma_wait_barrier<0>();
-    }
+  issue_b(0, 0);
+  if (nk > 1) issue_b(1, 1);
+  issue_a(0, 0);
+  if (nk > 1) {
+    issue_a(1, 1);
+    dma_wait_barrier<NJA>();  // in issue order only the token panel of slab 1 may still be under way
   } else {
-    issue_b(0, 0);
-    if (nk > 1) issue_b(1, 1);
-    issue_a(0, 0);
-    if (nk > 1) {
-      issue_a(1, 1);
-      dma_wait_barrier<NJA>();  // in issue order only the token panel of slab 1 may still be under way
-    } else {
-      dma_wait_barrier<0>();
-    }
+    dma_wait_barrier<0>();
   }
   if constexpr (Cfg::B_KMAJOR) {
     if (nk == 1 && kb.last_rows < kBK) kmajor_clear_tail(0);
@@ -649,15 +581,6 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
     for (; k0 < nk; k0 += 2) {
       kmajor_body(0, k0, false);
       if (k0 + 1 < nk) kmajor_body(1, k0 + 1, false);
-    }
-  } else if constexpr (Cfg::FIXED_SCHEDULE) {
-    for (; k0 + 3 < nk; k0 += 2) {
-      fixed_body(0, k0, true);
-      fixed_body(1, k0 + 1, true);
-    }
-    for (; k0 < nk; k0 += 2) {
-      fixed_body(0, k0, false);
-      if (k0 + 1 < nk) fixed_body(1, k0 + 1, false);
     }
   } else {
     for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches

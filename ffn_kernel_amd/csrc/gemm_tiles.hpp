@@ -59,10 +59,14 @@ inline hipError_t dispatch_tile(int tile, const GemmArgs& g, hipStream_t stream)
 // GEMMs on the 256x256 tile: when the tile count is not a multiple of the CU count, the last
 // round would run a few tiles on a few CUs for a full tile time (2064 tiles at M = 32768, N = 4096:
 // 8 rounds + 16 tiles).  Run the whole rounds with the big tile and the remainder in a second
-// launch: as 128x128 tiles (128 rows x 64 gate + 64 up columns for the SwiGLU kernel) of the same
-// schedule - same K order per output element, so the result does not depend on which launch computed
-// it - or, with GemmArgs::P_tail, on the big tile cut into K ranges plus a reduce pass (another
-// summation order for the rows of those tiles, a shorter tail: 0.20 -> 0.05 ms at the shape above).
+// launch: as 128x128 tiles (128 rows x 64 gate + 64 up columns for the SwiGLU kernel), or, with
+// GemmArgs::P_tail, on the big tile cut into K ranges plus a reduce pass (a shorter tail: 0.20 -> 0.05 ms
+// at the shape above).  Either way the rows of the remainder's tiles are summed in another fp32 order than
+// the rows of the whole rounds (32x32x16 MFMAs over 16-element K steps, or partial sums per K range,
+// against 16x16x32 MFMAs over 32-element steps): which launch a row falls into depends on the mask and on
+// the batch, so a row's result is reproducible for a given call but agrees between differently composed
+// calls only to fp32 summation accuracy - far inside the bf16 rounding of the output, and the bound the
+// batch-composition test states.
 template <class Tiles, class Big>
 inline hipError_t dispatch_big_tile_with_tail(const GemmArgs& g, hipStream_t stream) {
   using Small = typename Tiles::T2;

@@ -20,6 +20,7 @@ constexpr int kStreamMaxM = 64;
 struct TileChoice {
   int tile;    // TileId
   int splits;  // split-K factor (weight-gradient GEMM only)
+  bool tuned;  // the pair is a measured plan (as timed by the tuner), not the rules' guess
 };
 
 // Measured plans.  `python -m ffn_kernel_amd.tune --emit` times every candidate (tile x split-K factor)
@@ -29,9 +30,11 @@ struct TileChoice {
 // This is what the reference's find_spec/*.py searches and bf16_*.json tables are to its kernels
 // (find_spec/find.py:18-64, ffn_kernel/utils.py:3-5).
 enum TunedOp : int {
-  TUNED_PLAIN = 0,   // single-weight routed GEMM: k = contraction, n = output columns
+  TUNED_PLAIN = 0,   // MaskedLinear forward (gathered rows in, scattered rows out; whole-call timing): k = contraction, n = output columns
   TUNED_DUAL = 1,    // SwiGLU GEMM: k = contraction (d), n = output columns (h)
   TUNED_SPLITK = 2,  // weight-gradient GEMM: k = R (rows of the in-place operand), n = Cc
+  TUNED_DOWN = 3,    // MaskedFFN down projection (routed-order rows in, scattered out; stage timing): k = contraction (h), n = output columns (d)
+  TUNED_NONE = -1,   // a GEMM the tuner does not measure (the backward's dx GEMMs): rules only
 };
 struct TunedPlan {
   int op;            // TunedOp, -1 ends the table
@@ -50,9 +53,12 @@ inline const TunedPlan* tuned_plan(int op, int64_t M, int64_t k, int64_t n) {
 }
 
 // Routed GEMM over M rows and n_out output columns (K: the contraction, 0 = not known to the caller).
-inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual, int64_t K = 0, bool use_table = true) {
-  if (use_table && K > 0) {
-    if (const TunedPlan* t = tuned_plan(dual ? TUNED_DUAL : TUNED_PLAIN, M, K, n_out))
+// `op`: whose measured plans apply (TUNED_NONE: none; the tuner times each operation with its own gather /
+// scatter pattern and its own launches around the GEMM, so one operation's plan says nothing about another's).
+inline int pick_routed_tile(int64_t M, int64_t n_out, bool dual, int64_t K = 0, bool use_table = true,
+                            int op = TUNED_PLAIN) {
+  if (use_table && K > 0 && (dual || op != TUNED_NONE)) {
+    if (const TunedPlan* t = tuned_plan(dual ? TUNED_DUAL : op, M, K, n_out))
       if (dual || t->splits == 1) return t->tile;
   }
   auto tiles = [&](int tile) {
@@ -122,15 +128,15 @@ inline int pick_routed_splits(int64_t M, int64_t n_out, int64_t K, int tile) {
   return best;
 }
 
-inline RoutedPlan pick_routed_plan(int64_t M, int64_t n_out, int64_t K, bool use_table = true) {
+inline RoutedPlan pick_routed_plan(int64_t M, int64_t n_out, int64_t K, bool use_table = true, int op = TUNED_DOWN) {
   RoutedPlan p;
-  if (use_table)
-    if (const TunedPlan* t = tuned_plan(TUNED_PLAIN, M, K, n_out)) {
+  if (use_table && op != TUNED_NONE)
+    if (const TunedPlan* t = tuned_plan(op, M, K, n_out)) {
       p.tile = t->tile;
       p.splits = (K % 64 == 0 && M < 65536 && n_out % 4 == 0) ? t->splits : 1;
       return p;
     }
-  p.tile = pick_routed_tile(M, n_out, false, K, use_table);
+  p.tile = pick_routed_tile(M, n_out, false, K, use_table, op);
   p.splits = 1;
   if (M > 4096 || K % 64 != 0) return p;
   double best_cost = 0.0;
@@ -150,10 +156,12 @@ inline RoutedPlan pick_routed_plan(int64_t M, int64_t n_out, int64_t K, bool use
 // Weight-gradient GEMM: two [R, Cc] outputs, contraction over about M / 2 rows each.
 inline TileChoice pick_splitk_tile(int64_t M, int64_t R, int64_t Cc, bool use_table = true) {
   TileChoice c;
+  c.tuned = false;
   if (use_table)
     if (const TunedPlan* t = tuned_plan(TUNED_SPLITK, M, R, Cc)) {
       c.tile = t->tile;
       c.splits = t->splits;
+      c.tuned = true;
       return c;
     }
   // Large outputs: the 256x256 tile fills the chip on its own, no split needed (and the GEMM then

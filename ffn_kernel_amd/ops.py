@@ -9,6 +9,7 @@ Same class names, same positional signatures:
 from __future__ import annotations
 
 import contextlib
+import ctypes
 import threading
 
 import torch
@@ -99,8 +100,95 @@ def _wstrides(w: torch.Tensor):
     return sk, sn
 
 
-def masked_linear_forward(a: torch.Tensor, b1: torch.Tensor, b2: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
-    """c[m] = a[m] @ (b1 if mask[m] else b2).  Replaces _bf16_linear_forward (linear.py:418-452)."""
+class Routing:
+    """A row partition on the device: perm int32[M] (visual rows first, each group ascending) and
+    counts int32[2], as ffnk_route writes them.  One partition serves every operation that runs with the
+    same mask - the projections of a layer, a forward and its backward - where the reference re-tests the
+    mask inside every tile of every launch (linear.py:120-149, ffn.py:61-105)."""
+    __slots__ = ("perm", "counts", "M", "_struct")
+
+    def __init__(self, perm: torch.Tensor, counts: torch.Tensor):
+        self.perm, self.counts, self.M = perm, counts, perm.shape[0]
+        self._struct = _lib.RoutingStruct(perm.data_ptr(), counts.data_ptr())
+
+    def ref(self):
+        return ctypes.byref(self._struct)
+
+
+def route(mask: torch.Tensor) -> Routing:
+    """Partition the rows by mask on the mask's device and current stream (ffnk_route)."""
+    if not isinstance(mask, torch.Tensor) or mask.dtype != torch.bool or mask.dim() != 1 or not mask.is_cuda:
+        raise ValueError("route: mask must be a 1-D torch.bool tensor on a GPU")
+    M, dev = mask.shape[0], mask.device
+    mask = mask if mask.stride(0) == 1 or M <= 1 else mask.contiguous()
+    buf = torch.empty(M + 2, dtype=torch.int32, device=dev)
+    routing = Routing(buf[:M], buf[M:])
+    with _on_device(dev):
+        rc = _lib.load().ffnk_route(mask.data_ptr(), M, routing.perm.data_ptr(), routing.counts.data_ptr(), _stream_ptr(dev))
+    _lib.check(rc, "ffnk_route")
+    return routing
+
+
+class _RouteCache(threading.local):
+    """The last partition made on this thread and what it was made from."""
+    enabled = True
+    key = None
+    storage = None  # keeps the mask's memory alive, so that its address cannot be handed to another tensor
+    routing = None
+
+
+_route_cache = _RouteCache()
+_ROUTED_MIN_ROWS = 65  # up to 64 rows the weight-streaming kernels run, which read the mask themselves
+
+
+def set_route_cache(enabled: bool) -> bool:
+    """Switch the sharing of row partitions between calls on or off for this thread; returns the old setting."""
+    old = _route_cache.enabled
+    _route_cache.enabled = bool(enabled)
+    if not enabled:
+        _route_cache.key = _route_cache.storage = _route_cache.routing = None
+    return old
+
+
+def shared_routing(mask: torch.Tensor, M: int):
+    """The row partition for `mask`, made once and shared by the calls that follow with the same mask: the
+    operations of a transformer layer all route by one mask, and each would otherwise launch its own
+    partition kernel ahead of its GEMM.  The one-entry cache is keyed on the mask's memory (held alive by the
+    entry), its view, its version counter - every in-place write through torch bumps it, so a mask changed in
+    place is partitioned again - and the stream.  Returns None where no partition is shared: decode sizes,
+    the cache switched off, tensors without a version counter, a stream under graph capture (a captured
+    graph must not point at memory this cache may drop later)."""
+    if M < _ROUTED_MIN_ROWS or not _route_cache.enabled:
+        return None
+    dev = mask.device
+    try:
+        version = mask._version
+    except RuntimeError:  # inference tensors keep no version counter
+        return None
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    storage = mask.untyped_storage()
+    key = (storage.data_ptr(), mask.storage_offset(), mask.stride(0), M, version, dev.index, _stream_ptr(dev))
+    if _route_cache.key == key:
+        return _route_cache.routing
+    routing = route(mask)
+    _route_cache.key, _route_cache.storage, _route_cache.routing = key, storage, routing
+    return routing
+
+
+def _routing_arg(routing, mask: torch.Tensor, M: int):
+    """(Routing or None, its ffnk_routing_t* or None) for a call: the caller's, else the shared one."""
+    if routing is None:
+        routing = shared_routing(mask, M)
+    elif routing.M != M or routing.perm.device != mask.device:
+        raise ValueError(f"routing is for {routing.M} rows on {routing.perm.device}, the call has {M} on {mask.device}")
+    return routing, (routing.ref() if routing is not None else None)
+
+
+def masked_linear_forward(a: torch.Tensor, b1: torch.Tensor, b2: torch.Tensor, mask: torch.Tensor,
+                          routing: Routing | None = None) -> torch.Tensor:
+    """c[m] = a[m] @ (b1 if mask[m] else b2).  Replaces _bf16_linear_forward (linear.py:418-452).
+    routing: a partition of `mask` made by route(); None: the shared one (shared_routing)."""
     _require_cuda_bf16("a", a, 2)
     _require_cuda_bf16("b1", b1, 2)
     _require_cuda_bf16("b2", b2, 2)
@@ -122,17 +210,18 @@ def masked_linear_forward(a: torch.Tensor, b1: torch.Tensor, b2: torch.Tensor, m
         return c
     lib = _lib.load()
     with _on_device(dev):
+        routing, rt = _routing_arg(routing, mask, M)
         ws_bytes = _lib.workspace_bytes(_lib.OP_LINEAR_FWD, M, K, N)
         ws = _workspace(ws_bytes, dev)
-        rc = lib.ffnk_masked_linear_fwd(a.data_ptr(), a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(),
-                                        b2.data_ptr(), sk, sn, mask.data_ptr(), c.data_ptr(), N, M, K, N,
-                                        ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+        rc = lib.ffnk_masked_linear_fwd_routed(a.data_ptr(), a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(),
+                                               b2.data_ptr(), sk, sn, mask.data_ptr(), c.data_ptr(), N, M, K, N,
+                                               ws.data_ptr(), ws.numel(), _stream_ptr(dev), rt)
     _lib.check(rc, "ffnk_masked_linear_fwd")
     return c
 
 
 def masked_linear_backward(grad: torch.Tensor, a: torch.Tensor, b1: torch.Tensor, b2: torch.Tensor,
-                           mask: torch.Tensor):
+                           mask: torch.Tensor, routing: Routing | None = None):
     """(da, db1, db2) of MaskedLinear.  Replaces _bf16_linear_backward (linear.py:455-496);
     db1/db2 keep b1's strides as the reference's empty_like(b1) does (linear.py:475)."""
     _require_cuda_bf16("grad", grad, 2)
@@ -158,17 +247,18 @@ def masked_linear_backward(grad: torch.Tensor, a: torch.Tensor, b1: torch.Tensor
         return da, db1, db2
     lib = _lib.load()
     with _on_device(dev):
+        routing, rt = _routing_arg(routing, mask, M)
         ws_bytes = _lib.workspace_bytes(_lib.OP_LINEAR_BWD, M, K, N)
         ws = _workspace(ws_bytes, dev)
-        rc = lib.ffnk_masked_linear_bwd(grad.data_ptr(), grad.stride(0) if M > 1 else max(N, 1), a.data_ptr(),
-                                        a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(), b2.data_ptr(), sk, sn,
-                                        mask.data_ptr(), da.data_ptr(), K, db1.data_ptr(), db2.data_ptr(), dsk,
-                                        dsn, M, K, N, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+        rc = lib.ffnk_masked_linear_bwd_routed(grad.data_ptr(), grad.stride(0) if M > 1 else max(N, 1), a.data_ptr(),
+                                               a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(), b2.data_ptr(), sk, sn,
+                                               mask.data_ptr(), da.data_ptr(), K, db1.data_ptr(), db2.data_ptr(), dsk,
+                                               dsn, M, K, N, ws.data_ptr(), ws.numel(), _stream_ptr(dev), rt)
     _lib.check(rc, "ffnk_masked_linear_bwd")
     return da, db1, db2
 
 
-def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre: bool = False):
+def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre: bool = False, routing: Routing | None = None):
     """SwiGLU FFN routed by mask.  Replaces _bf16_ffn_forward + _bf16_linear_forward
     (ops.py:30-32, ffn.py:527-560).
 
@@ -210,21 +300,22 @@ def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre: bool = False):
     if save_pre and h > 0 and lib.ffnk_masked_ffn_can_save(M, d, h) and usk == 1 and dsk == 1:
         pre = torch.empty((M, 2 * h), device=dev, dtype=torch.bfloat16)
     with _on_device(dev):
+        routing, rt = _routing_arg(routing, mask, M)
         ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_FWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
         head = (a.data_ptr(), a.stride(0) if M > 1 else max(d, 1), ups[0].data_ptr(), ups[1].data_ptr(),
                 ups[2].data_ptr(), ups[3].data_ptr(), usk, usn, downs[0].data_ptr(), downs[1].data_ptr(), dsk, dsn,
                 mask.data_ptr(), out.data_ptr(), d)
-        tail = (M, d, h, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+        tail = (M, d, h, ws.data_ptr(), ws.numel(), _stream_ptr(dev), rt)
         if pre is None:
-            rc = lib.ffnk_masked_ffn_fwd(*head, *tail)
+            rc = lib.ffnk_masked_ffn_fwd_routed(*head, None, 0, *tail)
         else:
-            rc = lib.ffnk_masked_ffn_fwd_save(*head, pre.data_ptr(), 2 * h, *tail)
+            rc = lib.ffnk_masked_ffn_fwd_routed(*head, pre.data_ptr(), 2 * h, *tail)
     _lib.check(rc, "ffnk_masked_ffn_fwd")
     return (out, pre) if save_pre else out
 
 
-def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None):
+def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None, routing: Routing | None = None):
     """(da, dw1, dw2, dw3, du1, du2, du3) of MaskedFFN.  The reference stops at NotImplementedError
     here (ops.py:34-38); the decomposition follows its README sketch (README.md:159-172): routed
     GEMMs around one elementwise SwiGLU-gradient pass.  Weight gradients keep the strides of the
@@ -275,22 +366,33 @@ def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None):
         else:
             ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
+        routing, rt = _routing_arg(routing, mask, M)
         head = (grad.data_ptr(), grad.stride(0) if M > 1 else d, a.data_ptr(), a.stride(0) if M > 1 else d,
                 ups[0].data_ptr(), ups[1].data_ptr(), ups[2].data_ptr(), ups[3].data_ptr(), usk, usn,
                 downs[0].data_ptr(), downs[1].data_ptr(), dsk, dsn, mask.data_ptr())
         tail = (da.data_ptr(), d, dups[0].data_ptr(), dups[1].data_ptr(), dups[2].data_ptr(), dups[3].data_ptr(),
                 gusk, gusn, ddowns[0].data_ptr(), ddowns[1].data_ptr(), gdsk, gdsn, M, d, h, ws.data_ptr(), ws.numel(),
-                _stream_ptr(dev))
+                _stream_ptr(dev), rt)
         if pre is None:
-            rc = lib.ffnk_masked_ffn_bwd(*head, *tail)
+            rc = lib.ffnk_masked_ffn_bwd_routed(*head, None, 0, *tail)
         else:
             if pre.shape != (M, 2 * h) or pre.dtype != torch.bfloat16 or pre.device != dev or pre.stride(1) != 1:
                 raise ValueError(f"pre must be a bf16 [{M}, {2 * h}] tensor on {dev} with contiguous rows")
-            rc = lib.ffnk_masked_ffn_bwd_saved(*head, pre.data_ptr(), pre.stride(0) if M > 1 else 2 * h, *tail)
+            rc = lib.ffnk_masked_ffn_bwd_routed(*head, pre.data_ptr(), pre.stride(0) if M > 1 else 2 * h, *tail)
     _lib.check(rc, "ffnk_masked_ffn_bwd")
     dw1, dw3, du1, du3 = dups
     dw2, du2 = ddowns
     return da, dw1, dw2, dw3, du1, du2, du3
+
+
+def _forward_routing(mask):
+    """The shared partition for a well-formed mask (None otherwise: the forward's own checks then report it)."""
+    if isinstance(mask, torch.Tensor) and mask.dtype == torch.bool and mask.dim() == 1 and mask.is_cuda:
+        m = mask if mask.stride(0) == 1 or mask.shape[0] <= 1 else None
+        if m is not None:
+            with _on_device(mask.device):
+                return shared_routing(m, m.shape[0])
+    return None
 
 
 class _GradMode(threading.local):
@@ -308,14 +410,17 @@ class MaskedLinear(Function):
     def forward(ctx, a, b1, b2, mask):
         ctx.save_for_backward(a, mask)
         ctx.b1, ctx.b2 = b1, b2
-        return masked_linear_forward(a, b1, b2, mask)
+        # the partition the forward runs with serves the backward too (autograd refuses a saved mask that
+        # was changed in place, so it cannot go stale)
+        ctx.routing = _forward_routing(mask)
+        return masked_linear_forward(a, b1, b2, mask, routing=ctx.routing)
 
     @staticmethod
     @once_differentiable
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad):
         a, mask = ctx.saved_tensors
-        da, db1, db2 = masked_linear_backward(grad, a, ctx.b1, ctx.b2, mask)
+        da, db1, db2 = masked_linear_backward(grad, a, ctx.b1, ctx.b2, mask, routing=ctx.routing)
         return da, db1, db2, None
 
 
@@ -337,10 +442,11 @@ class MaskedFFN(Function):
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, a, w1, w2, w3, u1, u2, u3, mask):
         ctx.weights = (w1, w2, w3, u1, u2, u3)
+        ctx.routing = _forward_routing(mask)
         if _grad_mode.enabled and any(ctx.needs_input_grad):
-            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre=True)
+            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre=True, routing=ctx.routing)
         else:
-            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask), None
+            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, routing=ctx.routing), None
         ctx.has_pre = pre is not None
         if pre is None:
             ctx.save_for_backward(a, mask)
@@ -354,4 +460,4 @@ class MaskedFFN(Function):
     def backward(ctx, grad):
         a, mask = ctx.saved_tensors[:2]
         pre = ctx.saved_tensors[2] if ctx.has_pre else None
-        return (*masked_ffn_backward(grad, a, *ctx.weights, mask, pre=pre), None)
+        return (*masked_ffn_backward(grad, a, *ctx.weights, mask, pre=pre, routing=ctx.routing), None)

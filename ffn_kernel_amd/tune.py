@@ -38,7 +38,7 @@ from .ops import masked_linear_backward, masked_linear_forward
 
 TILES = {0: "256x256/8w", 1: "256x256/4w", 2: "128x128/4w", 3: "small/4w", 4: "128x128/ring4"}
 SPLITS = (1, 2, 3, 4, 6, 7, 8, 12, 14, 16)
-TUNED_PLAIN, TUNED_DUAL, TUNED_SPLITK = 0, 1, 2
+TUNED_PLAIN, TUNED_DUAL, TUNED_SPLITK, TUNED_DOWN = 0, 1, 2, 3  # TunedOp in csrc/tile_table.hpp
 GEN_PATH = Path(__file__).resolve().parent / "csrc" / "tile_table_gen.hpp"
 
 # M buckets [lo, hi]; each is measured at its upper end.  Below 65 rows the FFN runs the streaming kernels.
@@ -306,7 +306,7 @@ def plans_from(records, margin):
                 out.append((TUNED_DUAL, r["m_lo"], r["m_hi"], r["d"], r["h"], tile, 1))
             key, _ = _select(r["rules_down_ms"], r["down_ms"], margin)
             if key is not None:
-                out.append((TUNED_PLAIN, r["m_lo"], r["m_hi"], r["h"], r["d"], key[0], key[1]))
+                out.append((TUNED_DOWN, r["m_lo"], r["m_hi"], r["h"], r["d"], key[0], key[1]))
         elif r["op"] == "linear_fwd":
             key, _ = _select(r["rules_ms"], r["ms"], margin)
             if key is not None:
@@ -316,7 +316,8 @@ def plans_from(records, margin):
             if s is not None:
                 tile = {(256, 256): 0, (128, 128): 2}.get((r["rules"]["block_m"], r["rules"]["block_n"]), 2)
                 out.append((TUNED_SPLITK, r["m_lo"], r["m_hi"], r["N"], r["K"], tile, s))  # R = N, Cc = K (dW stored [N, K])
-    # one entry per key: a linear layer and an FFN's down projection can share (k, n); keep the first
+    # one entry per key (the operation is part of it: a linear layer and an FFN's down projection of the
+    # same extents are different kernels and keep their own plans)
     seen, uniq = set(), []
     for e in sorted(out):
         if e[:5] not in seen:

@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define FFNK_VERSION 100
+#define FFNK_VERSION 101
 
 #if defined(__GNUC__)
 #define FFNK_API __attribute__((visibility("default")))
@@ -93,6 +93,20 @@ FFNK_API const char* ffnk_last_error(void);
  */
 FFNK_API int ffnk_route(const uint8_t* mask, int64_t M, int32_t* perm, int32_t* counts, void* stream);
 
+/*
+ * A row partition made earlier by ffnk_route for the same mask and M, handed to the *_routed entry points
+ * below so that the operations of a layer - and a forward and its backward - share one partition instead
+ * of each running its own.  perm: int32[M], counts: int32[2], both DEVICE memory that holds ffnk_route's
+ * output by the time the call's kernels run (same stream, or ordered by the caller) and stays unchanged
+ * until they have finished.  The struct itself is host memory, read during the call.  The reference has
+ * nothing to share here: its kernels re-test the mask inside every tile of every launch
+ * (ffn_kernel/linear.py:120-149, ffn_kernel/ffn.py:61-105).
+ */
+typedef struct ffnk_routing_t {
+  const int32_t* perm;
+  const int32_t* counts;
+} ffnk_routing_t;
+
 /* Bytes of scratch the op needs for these extents (0 is a valid answer).
  * Returns (size_t)-1 for an unknown op or invalid extents. */
 FFNK_API size_t ffnk_workspace_bytes(int op, int64_t M, int64_t K, int64_t N);
@@ -141,6 +155,17 @@ FFNK_API int ffnk_masked_linear_fwd(const uint16_t* x, int64_t x_stride_m,
                            uint16_t* y, int64_t y_stride_m,
                            int64_t M, int64_t K, int64_t N,
                            void* ws, size_t ws_bytes, void* stream);
+
+/* ffnk_masked_linear_fwd with the row partition handed in (routing == NULL: exactly ffnk_masked_linear_fwd).
+ * `mask` is still required: the weight-streaming kernels for M <= 64 and the any-stride kernels read it
+ * themselves and ignore `routing`.  What it replaces: the per-tile mask test of ffn_kernel/linear.py:120-149. */
+FFNK_API int ffnk_masked_linear_fwd_routed(const uint16_t* x, int64_t x_stride_m,
+                                  const uint16_t* Wv, const uint16_t* Wt,
+                                  int64_t w_stride_k, int64_t w_stride_n,
+                                  const uint8_t* mask,
+                                  uint16_t* y, int64_t y_stride_m,
+                                  int64_t M, int64_t K, int64_t N,
+                                  void* ws, size_t ws_bytes, void* stream, const ffnk_routing_t* routing);
 
 /*
  * MaskedFFN forward — replaces _bf16_ffn_forward followed by _bf16_linear_forward
@@ -224,6 +249,20 @@ FFNK_API int ffnk_masked_linear_bwd(const uint16_t* g, int64_t g_stride_m,
                            int64_t M, int64_t K, int64_t N,
                            void* ws, size_t ws_bytes, void* stream);
 
+/* ffnk_masked_linear_bwd with the row partition handed in (routing == NULL: exactly ffnk_masked_linear_bwd);
+ * a backward can reuse the partition its forward ran with.  Replaces the mask tests of
+ * ffn_kernel/linear.py:288-291, 299-313, 398-403. */
+FFNK_API int ffnk_masked_linear_bwd_routed(const uint16_t* g, int64_t g_stride_m,
+                                  const uint16_t* x, int64_t x_stride_m,
+                                  const uint16_t* Wv, const uint16_t* Wt,
+                                  int64_t w_stride_k, int64_t w_stride_n,
+                                  const uint8_t* mask,
+                                  uint16_t* dx, int64_t dx_stride_m,
+                                  uint16_t* dWv, uint16_t* dWt,
+                                  int64_t dw_stride_k, int64_t dw_stride_n,
+                                  int64_t M, int64_t K, int64_t N,
+                                  void* ws, size_t ws_bytes, void* stream, const ffnk_routing_t* routing);
+
 /*
  * MaskedFFN backward.  The reference declares it but raises NotImplementedError
  * (ffn_kernel/ops.py:34-38); its README (README.md:159-172) sketches the decomposition used
@@ -306,6 +345,42 @@ FFNK_API int ffnk_masked_ffn_bwd_saved(const uint16_t* g, int64_t g_stride_m,
                               int64_t ddown_stride_k, int64_t ddown_stride_n,
                               int64_t M, int64_t d, int64_t h,
                               void* ws, size_t ws_bytes, void* stream);
+
+/*
+ * The MaskedFFN forward and backward with the row partition handed in (see ffnk_routing_t; routing == NULL:
+ * a route launch at the head of the call, as in the plain entry points).  `pre` is optional in both:
+ * forward: NULL = ffnk_masked_ffn_fwd, else ffnk_masked_ffn_fwd_save; backward: NULL = ffnk_masked_ffn_bwd
+ * (recompute), else ffnk_masked_ffn_bwd_saved.  Replaces the per-tile mask tests of ffn_kernel/ffn.py:61-105
+ * and ffn_kernel/linear.py:120-149.
+ */
+FFNK_API int ffnk_masked_ffn_fwd_routed(const uint16_t* x, int64_t x_stride_m,
+                               const uint16_t* W1, const uint16_t* W3,
+                               const uint16_t* U1, const uint16_t* U3,
+                               int64_t up_stride_k, int64_t up_stride_n,
+                               const uint16_t* W2, const uint16_t* U2,
+                               int64_t down_stride_k, int64_t down_stride_n,
+                               const uint8_t* mask,
+                               uint16_t* out, int64_t out_stride_m,
+                               uint16_t* pre, int64_t pre_stride_m,
+                               int64_t M, int64_t d, int64_t h,
+                               void* ws, size_t ws_bytes, void* stream, const ffnk_routing_t* routing);
+
+FFNK_API int ffnk_masked_ffn_bwd_routed(const uint16_t* g, int64_t g_stride_m,
+                               const uint16_t* x, int64_t x_stride_m,
+                               const uint16_t* W1, const uint16_t* W3,
+                               const uint16_t* U1, const uint16_t* U3,
+                               int64_t up_stride_k, int64_t up_stride_n,
+                               const uint16_t* W2, const uint16_t* U2,
+                               int64_t down_stride_k, int64_t down_stride_n,
+                               const uint8_t* mask,
+                               const uint16_t* pre, int64_t pre_stride_m,
+                               uint16_t* dx, int64_t dx_stride_m,
+                               uint16_t* dW1, uint16_t* dW3, uint16_t* dU1, uint16_t* dU3,
+                               int64_t dup_stride_k, int64_t dup_stride_n,
+                               uint16_t* dW2, uint16_t* dU2,
+                               int64_t ddown_stride_k, int64_t ddown_stride_n,
+                               int64_t M, int64_t d, int64_t h,
+                               void* ws, size_t ws_bytes, void* stream, const ffnk_routing_t* routing);
 
 #ifdef __cplusplus
 }

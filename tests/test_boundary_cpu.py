@@ -95,8 +95,16 @@ def test_tile_table_entries():
     assert _lib.tile_config(_lib.OP_LINEAR_FWD, 1, 4096, 4096)["path"] == _lib.PATH_STREAM
     assert _lib.tile_config(_lib.OP_LINEAR_FWD, 64, 4096, 4096)["path"] == _lib.PATH_STREAM
     assert _lib.tile_config(_lib.OP_LINEAR_FWD, 64, 4096, 4100)["path"] == _lib.PATH_MFMA_TILED  # ragged N
+    # the factor reported is the one launched: the fused dx / dW launch of the usual layout runs cfg3's
+    # weight-gradient GEMM unsplit, whatever the stand-alone GEMM's rule would pick; a forced factor is kept
     dw = _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)
-    assert dw["split_k"] > 1
+    assert dw["split_k"] == 1
+    lib = _lib.load()
+    try:
+        lib.ffnk_debug_force_splits(4)
+        assert _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)["split_k"] == 4
+    finally:
+        lib.ffnk_debug_force_splits(-1)
     with pytest.raises(ValueError):
         _lib.tile_config(77, 1, 1, 1)
 
@@ -192,9 +200,9 @@ def test_reference_import_name_resolves():
 
 
 def test_row_limit_is_what_one_route_launch_handles():
-    assert _lib.workspace_bytes(_lib.OP_LINEAR_FWD, 1 << 22, 64, 64) > 0
+    assert _lib.workspace_bytes(_lib.OP_LINEAR_FWD, 1 << 24, 64, 64) > 0
     with pytest.raises(ValueError):
-        _lib.workspace_bytes(_lib.OP_LINEAR_FWD, (1 << 22) + 1, 64, 64)
+        _lib.workspace_bytes(_lib.OP_LINEAR_FWD, (1 << 24) + 1, 64, 64)
 
 
 def test_measured_plans_are_consulted_before_the_rules():
@@ -215,15 +223,41 @@ def test_measured_plans_are_consulted_before_the_rules():
                 assert (cfg["block_m"], cfg["waves_m"] * cfg["waves_n"]) == (geom[tile][0], geom[tile][2]), (op, hi, k, n, cfg)
             checked += 1
         elif op == tune.TUNED_PLAIN:
+            cfg = _lib.tile_config(_lib.OP_LINEAR_FWD, hi, k, n)
+            if cfg["path"] == _lib.PATH_MFMA_TILED:
+                assert cfg["split_k"] == splits, (op, hi, k, n, cfg)
+                if tile in geom and splits == 1:
+                    assert (cfg["block_m"], cfg["block_n"]) == geom[tile][:2]
+                checked += 1
+            # a linear layer's plan is not an FFN down projection's, even at the same extents
+            if not any(e[0] == tune.TUNED_DOWN and e[3:5] == (k, n) and e[1] <= hi <= e[2] for e in entries):
+                try:
+                    lib.ffnk_debug_force_tile(-2)
+                    rules = _lib.tile_config(_lib.OP_FFN_DOWN, hi, n, k)
+                finally:
+                    lib.ffnk_debug_force_tile(-1)
+                assert _lib.tile_config(_lib.OP_FFN_DOWN, hi, n, k) == rules, (hi, k, n)
+        elif op == tune.TUNED_DOWN:
             cfg = _lib.tile_config(_lib.OP_FFN_DOWN, hi, n, k)  # FFN extents: K = d = output columns, N = h = contraction
             if cfg["path"] == _lib.PATH_MFMA_TILED:
                 assert cfg["split_k"] == splits, (op, hi, k, n, cfg)
                 if tile in geom:
                     assert (cfg["block_m"], cfg["block_n"]) == geom[tile][:2]
                 checked += 1
+        elif op == tune.TUNED_SPLITK:
+            # k = R = N, n = Cc = K of the MaskedLinear backward; the measured factor is launched as it is,
+            # also where the fused launch's own cost model would have chosen otherwise
+            for M in (hi, (lo + hi) // 2):
+                cfg = _lib.tile_config(_lib.OP_BWD_DW, M, n, k)
+                assert cfg["split_k"] == splits, (op, M, k, n, cfg)
+                if tile in geom:
+                    assert (cfg["block_m"], cfg["block_n"]) == geom[tile][:2]
+            checked += 1
     assert checked > 0 or not entries
+    ops_seen = {e[0] for e in entries}
+    assert ops_seen <= {tune.TUNED_PLAIN, tune.TUNED_DUAL, tune.TUNED_SPLITK, tune.TUNED_DOWN}
     if entries:
-        op, lo, hi, k, n, tile, splits = next((e for e in entries if e[0] == tune.TUNED_PLAIN), entries[0])
+        op, lo, hi, k, n, tile, splits = next((e for e in entries if e[0] == tune.TUNED_DOWN), entries[0])
         try:
             assert lib.ffnk_debug_force_tile(-2) == -1
             rules = _lib.tile_config(_lib.OP_FFN_DOWN, hi, n, k)

@@ -188,7 +188,114 @@ def test_cfg5_decode_fullsize(dev, M, kind):
             W[k] = torch.full_like(W[k], float("nan"))
         out2 = MaskedFFN.apply(*wl.FFNWorkload("p", w.x, W, w.mask).op_args())
         assert torch.equal(out2, out)
+    # every row against the select form in fp32 library matmuls on the GPU, at the tolerance of the tiled path
+    assert_close(out, _ffn_select_fp32(w.x, w.W, w.mask), f"decode M={M} {kind}, every row")
     # one row in double precision
     wc = wl.cfg5_ffn_decode(M, kind)
     sub = wl.FFNWorkload("r", wc.x[:1], wc.W, wc.mask[:1])
     assert_close(out[:1], cref.ffn_fwd(sub.x, sub.W, sub.mask, round_mid=True), "decode row 0")
+
+
+def _ffn_select_fp32(x, W, mask):
+    """The reference module's maths (test_ffn.py:43-47) in row-select form: fp32 library matmuls on the
+    GPU, the intermediate rounded to bf16 once as the kernels store it.  Returns float64 on the host."""
+    xf = x.float()
+    ref = torch.zeros(x.shape[0], W["w2"].shape[0], device=x.device, dtype=torch.float32)
+    for sel, (k1, k2, k3) in ((mask, ("w1", "w2", "w3")), (~mask, ("u1", "u2", "u3"))):
+        if not bool(sel.any()):
+            continue
+        t1 = xf[sel] @ W[k1].float().T
+        t3 = xf[sel] @ W[k3].float().T
+        hmid = (t1 * torch.sigmoid(t1) * t3).to(torch.bfloat16).float()
+        ref[sel] = hmid @ W[k2].float().T
+    return ref.double().cpu()
+
+
+def _span_mask(M, seq, spans, span, seed):
+    """The reference's generate_mask idea (test_linear.py:15-21) per sequence: `spans` contiguous visual
+    spans of `span` tokens at seeded, non-overlapping positions in every `seq`-token sequence."""
+    gen = torch.Generator().manual_seed(seed)
+    mask = torch.zeros(M, dtype=torch.bool)
+    for s0 in range(0, M, seq):
+        slots = torch.randperm(seq // span, generator=gen)[:spans]
+        for k in slots.tolist():
+            mask[s0 + k * span:s0 + (k + 1) * span] = True
+    return mask
+
+
+def test_linear_fwd_bwd_at_the_end_of_the_reference_sweep(dev):
+    """MaskedLinear forward and backward at M = 63488, K = N = 1024: the last point of the reference's own
+    --check sweep (test_linear.py:88, seq_len = 2048 * 31), past the 32768 rows of the largest benchmark
+    shape.  Every row and every gradient against fp32 library matmuls of the select form on the GPU."""
+    note("linear fwd+bwd M=63488 K=N=1024")
+    M, K, N = 63488, 1024, 1024
+    mask = _span_mask(M, 2048, 1, 1024, seed=3)   # one 1024-token image per 2048-token sequence, as test_linear.py:11-21
+    w = wl.make_linear("sweep-end", M, K, N, mask, seed=4).to(dev)
+    g = torch.Generator(device=dev).manual_seed(5)
+    grad = torch.randn(M, N, device=dev, generator=g).to(torch.bfloat16)
+    x = w.x.clone().requires_grad_(True)
+    wv = w.Wv.clone().requires_grad_(True)
+    wt = w.Wt.clone().requires_grad_(True)
+    y = MaskedLinear.apply(x, wv.T, wt.T, w.mask)
+    y.backward(grad)
+    m2 = w.mask[:, None]
+    xf, gf = w.x.float(), grad.float()
+    assert_close(y, torch.where(m2, xf @ w.Wv.float().T, xf @ w.Wt.float().T).double().cpu(), "y")
+    assert_close(x.grad, torch.where(m2, gf @ w.Wv.float(), gf @ w.Wt.float()).double().cpu(), "dx")
+    # weight gradients sum 31744 rows each: compare at the scale of the sum (what a bf16 result can hold)
+    for name, got, sel in (("dWv", wv.grad, w.mask), ("dWt", wt.grad, ~w.mask)):
+        ref = (gf[sel].T @ xf[sel]).double().cpu()
+        rep = om.error_report(got.float().cpu(), ref)
+        assert rep["rel_l2"] <= om.REL_L2_TOL and rep["max_excess"] <= 1.0, (name, rep)
+
+
+def test_ffn_fwd_at_the_last_key_of_the_reference_tables(dev):
+    """MaskedFFN forward at M = 131072, d = 1024, h = 2048: the last key of the reference's largest tile
+    table (ffn_kernel/bf16_ffn_bwd.json) at test_ffn.py:87-88's layer.  Every row against fp32 library
+    matmuls of the select form on the GPU."""
+    note("ffn fwd M=131072 d=1024 h=2048")
+    M, d, h = 131072, 1024, 2048
+    mask = _span_mask(M, 2048, 2, 576, seed=6)
+    w = wl.make_ffn("tables-end", M, d, h, mask, seed=7).to(dev)
+    out = MaskedFFN.apply(*w.op_args())
+    for lo in range(0, M, 32768):   # the fp32 reference in four pieces
+        sl = slice(lo, lo + 32768)
+        assert_close(out[sl], _ffn_select_fp32(w.x[sl], w.W, w.mask[sl]), f"rows {lo}..{lo + 32768}")
+
+
+def test_gather_offsets_past_32_bits_take_the_staged_path(dev):
+    """Token rows whose byte offsets from the first row do not fit 32 bits (here: 40000 rows at a row stride
+    of 65536 elements, a view into a wider buffer) cannot use the global->LDS loads, which address with
+    32-bit offsets; the forward and the backward must notice and run their register-staged loops - at size,
+    with the rows that need the upper offset bits among those checked."""
+    note("linear fwd+bwd, row stride 65536 elements, M=40000")
+    M, K, N, ld = 40000, 256, 512, 65536
+    assert M * ld * 2 >= 1 << 32
+    gen = torch.Generator().manual_seed(8)
+    mask = (torch.rand(M, generator=gen) < 0.5).to(dev)
+    g = torch.Generator(device=dev).manual_seed(9)
+    wide = torch.empty(M, ld, device=dev, dtype=torch.bfloat16)
+    wide[:, :K] = torch.randn(M, K, device=dev, generator=g).to(torch.bfloat16)
+    x = wide[:, :K]
+    assert x.stride(0) == ld
+    Wv = (torch.randn(N, K, device=dev, generator=g) * 0.05).to(torch.bfloat16)
+    Wt = (torch.randn(N, K, device=dev, generator=g) * 0.05).to(torch.bfloat16)
+    y = MaskedLinear.apply(x, Wv.T, Wt.T, mask)
+    xf = x.float()
+    ref = torch.where(mask[:, None], xf @ Wv.float().T, xf @ Wt.float().T)
+    assert_close(y, ref.double().cpu(), "strided x, forward")
+    del wide, x, xf, ref
+    torch.cuda.empty_cache()
+    # the backward gathers grad rows the same way: a wide grad buffer
+    gwide = torch.empty(M, ld, device=dev, dtype=torch.bfloat16)
+    gwide[:, :N] = torch.randn(M, N, device=dev, generator=g).to(torch.bfloat16)
+    grad = gwide[:, :N]
+    xs = torch.randn(M, K, device=dev, generator=g).to(torch.bfloat16)
+    from ffn_kernel_amd import masked_linear_backward
+    dx, dwv, dwt = masked_linear_backward(grad, xs, Wv.T, Wt.T, mask)
+    gf = grad.float()
+    assert_close(dx, torch.where(mask[:, None], gf @ Wv.float(), gf @ Wt.float()).double().cpu(), "strided grad, dx")
+    for name, got, sel in (("dWv", dwv, mask), ("dWt", dwt, ~mask)):
+        ref = (xs.float()[sel].T @ gf[sel]).double().cpu()   # logical [K, N]
+        rep = om.error_report(got.float().cpu(), ref)
+        assert rep["rel_l2"] <= om.REL_L2_TOL and rep["max_excess"] <= 1.0, (name, rep)

@@ -20,7 +20,8 @@ pytestmark = pytest.mark.gpu
 
 
 # ------------------------------------------------------------------ routing (integer, bit-exact)
-@pytest.mark.parametrize("M", [0, 1, 2, 15, 16, 17, 63, 64, 65, 255, 4095, 4096, 4097, 10000, 32768, 100003])
+@pytest.mark.parametrize("M", [0, 1, 2, 15, 16, 17, 63, 64, 65, 255, 4095, 4096, 4097, 10000, 32768, 100003, 262144, 262145,
+                               600001])  # past 262144 rows a block of the partition kernel places several 1024-row chunks
 @pytest.mark.parametrize("p", [0.0, 0.5, 1.0])
 def test_route_bit_exact(dev, M, p):
     note(f"route M={M} p={p}")
@@ -922,3 +923,106 @@ def test_ffn_bwd_lean_workspace_is_enough_and_changes_nothing(dev, M, d, h, layo
         assert torch.equal(a, b), name
     if d % 64 == 0 and h % 64 == 0:
         assert sizes[0] < worst  # weights and intermediates read in place: no room for copies or transposes
+
+
+# ------------------------------------------------------------------ one row partition shared by several calls
+def _count_route_launches(monkeypatch):
+    """Count the partitions made from Python (ops.route) while the block runs."""
+    from ffn_kernel_amd import ops
+    calls = []
+    real = ops.route
+    monkeypatch.setattr(ops, "route", lambda mask: (calls.append(mask.shape[0]), real(mask))[1])
+    return calls
+
+
+def test_routing_is_shared_between_the_calls_of_a_layer_and_with_the_backward(dev, monkeypatch):
+    """The operations of a layer run with one mask: the partition is made once (ops.shared_routing) and handed
+    to every call through the *_routed entry points; a forward's partition serves its backward.  Results are
+    those of calls that each partition the rows themselves, bit for bit."""
+    note("shared routing: linear fwd + bwd + ffn fwd + bwd on one mask")
+    from ffn_kernel_amd import ops
+    M, K, N, d, h = 700, 256, 384, 256, 512
+    gen = torch.Generator().manual_seed(41)
+    mask = (torch.rand(M, generator=gen) < 0.4).to(dev)
+    lw = wl.make_linear("l", M, K, N, mask.cpu(), seed=42, with_grad=True).to(dev)
+    fw = wl.make_ffn("f", M, d, h, mask.cpu(), seed=43).to(dev)
+
+    def layer():
+        x = lw.x.clone().requires_grad_(True)
+        y = MaskedLinear.apply(x, lw.Wv.T, lw.Wt.T, mask)
+        y.backward(lw.grad)
+        xf = fw.x.clone().requires_grad_(True)
+        o = MaskedFFN.apply(xf, *fw.op_args()[1:7], mask)
+        o.backward(torch.ones_like(o))
+        return y.detach(), x.grad, o.detach(), xf.grad
+
+    old = ops.set_route_cache(False)
+    try:
+        want = layer()
+    finally:
+        ops.set_route_cache(old)
+    ops.set_route_cache(False)
+    ops.set_route_cache(True)  # start from an empty cache
+    calls = _count_route_launches(monkeypatch)
+    got = layer()
+    assert calls == [M], f"one partition for the whole layer, got {calls}"
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    # an explicit partition works the same and bypasses the cache
+    r = ops.route(mask)
+    assert torch.equal(ops.masked_linear_forward(lw.x, lw.Wv.T, lw.Wt.T, mask, routing=r), want[0])
+    with pytest.raises(ValueError, match="rows"):
+        ops.masked_linear_forward(lw.x[:600], lw.Wv.T, lw.Wt.T, mask[:600], routing=r)
+
+
+def test_a_mask_changed_in_place_is_partitioned_again(dev, monkeypatch):
+    """The shared partition is keyed on the mask's memory, view and version counter: a write into the mask,
+    a different view of it, or another mask at the same extents each get their own partition, and the results
+    follow the mask as it is at the time of the call."""
+    note("shared routing: stale partitions cannot be hit")
+    from ffn_kernel_amd import ops
+    M, K, N = 900, 128, 256
+    gen = torch.Generator().manual_seed(51)
+    mask = (torch.rand(M, generator=gen) < 0.5).to(dev)
+    w = wl.make_linear("l", M, K, N, mask.cpu(), seed=52).to(dev)
+
+    def ref(m):
+        return torch.where(m[:, None], w.x.float() @ w.Wv.float().T, w.x.float() @ w.Wt.float().T).double().cpu()
+
+    ops.set_route_cache(False)
+    ops.set_route_cache(True)
+    calls = _count_route_launches(monkeypatch)
+    assert_close(MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, mask), ref(mask), "first mask")
+    MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, mask)
+    assert len(calls) == 1
+    mask[:300] = ~mask[:300]                      # in place: same memory, new version
+    assert_close(MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, mask), ref(mask), "mask changed in place")
+    assert len(calls) == 2
+    other = ~mask                                  # another tensor
+    assert_close(MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, other), ref(other), "another mask")
+    assert len(calls) == 3
+    both = torch.cat([mask, other])
+    view = both[M:]                                # same storage as `both`, other offset
+    assert_close(MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, both[:M]), ref(mask), "view at offset 0")
+    assert_close(MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, view), ref(other), "view at offset M")
+    assert len(calls) == 5
+    # decode sizes never share a partition (the streaming kernels read the mask themselves)
+    MaskedLinear.apply(w.x[:40], w.Wv.T, w.Wt.T, mask[:40])
+    assert len(calls) == 5
+
+
+def test_routed_entry_points_reject_half_a_partition(dev):
+    note("ffnk_masked_linear_fwd_routed with perm but no counts")
+    lib = _lib.load()
+    M, K, N = 128, 64, 64
+    x = torch.zeros(M, K, device=dev, dtype=torch.bfloat16)
+    W = torch.zeros(N, K, device=dev, dtype=torch.bfloat16)
+    y = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+    mask = torch.zeros(M, dtype=torch.bool, device=dev)
+    perm = torch.zeros(M, dtype=torch.int32, device=dev)
+    ws = torch.empty(_lib.workspace_bytes(_lib.OP_LINEAR_FWD, M, K, N), dtype=torch.uint8, device=dev)
+    half = _lib.RoutingStruct(perm.data_ptr(), None)
+    rc = lib.ffnk_masked_linear_fwd_routed(x.data_ptr(), K, W.data_ptr(), W.data_ptr(), 1, K, mask.data_ptr(), y.data_ptr(),
+                                           N, M, K, N, ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream,
+                                           ctypes.byref(half))
+    assert rc == -1  # FFNK_E_NULL

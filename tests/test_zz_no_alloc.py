@@ -39,12 +39,22 @@ def _static(w):
     lib = _lib.load()
     M, d = w.x.shape
     out = torch.full((M, d), float("nan"), device=w.x.device, dtype=torch.bfloat16)
+    stream = torch.cuda.current_stream().cuda_stream
+    # Once untimed: the first call on a GPU looks the scratch array's address up, and the runtime loads a
+    # kernel's code the first time it is launched.  The call that counts must leave both of torch's
+    # counters and the device's own free-memory figure where they were - the latter also sees a hipMalloc
+    # made inside the library, which torch's allocator statistics would not.
+    _lib.check(lib.ffnk_masked_ffn_fwd_static(*_args(w, out), stream), "ffnk_masked_ffn_fwd_static")
+    torch.cuda.synchronize()
+    out.fill_(float("nan"))
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
-    rc = lib.ffnk_masked_ffn_fwd_static(*_args(w, out), torch.cuda.current_stream().cuda_stream)
+    free_before = torch.cuda.mem_get_info()[0]
+    rc = lib.ffnk_masked_ffn_fwd_static(*_args(w, out), stream)
     _lib.check(rc, "ffnk_masked_ffn_fwd_static")
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before, "device memory was allocated during the call"
     return out
 
 
@@ -83,3 +93,15 @@ def test_static_scratch_forward_rejects_what_does_not_fit(dev):
     assert rc == -5  # FFNK_E_WORKSPACE
     with pytest.raises(ValueError, match="static"):
         _lib.check(rc, "ffnk_masked_ffn_fwd_static")
+
+
+def test_static_scratch_is_looked_up_on_the_device_of_the_output(dev):
+    """The scratch array's address is taken on the GPU that holds `out`, whatever the calling thread's
+    current device: an output that is not device memory is refused before anything is launched."""
+    note("ffnk_masked_ffn_fwd_static with a host output pointer")
+    lib = _lib.load()
+    host = torch.empty(64, 64, dtype=torch.bfloat16)
+    rc = lib.ffnk_masked_ffn_fwd_static(0, 64, 0, 0, 0, 0, 1, 64, 0, 0, 1, 64, 0, host.data_ptr(), 64, 64, 64, 64, 0)
+    assert rc == -1  # FFNK_E_NULL
+    torch.cuda.synchronize()  # the refused query left no error behind for the next call
+    assert torch.zeros(4, device=dev).sum().item() == 0
