@@ -510,7 +510,8 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->group_m = dual ? 8 : 4;
   out->split_k = splits;
   out->direct_lds = direct ? 1 : 0;
-  out->lds_stages = (tile == TILE_128x128_R4 && out->direct_lds) ? 4 : 2;
+  // 4: ring of four stages (128x128); 3: token panel in three stages, weight panel in two (single-weight 256x256 tiles)
+  out->lds_stages = !out->direct_lds ? 2 : tile == TILE_128x128_R4 ? 4 : (is_big_tile(tile) && !dual) ? 3 : 2;
   if (op == FFNK_OP_FFN_DOWN && !stream) out->split_k = tiled_down_splits(M, K, N);
   if (op == FFNK_OP_LINEAR_FWD && linear_stream_kind(M, K, N)) {
     out->path = FFNK_PATH_STREAM;

@@ -131,10 +131,13 @@ struct RoutedGemmCfg {
   // More than two stages: a ring of K slabs with the loads STAGES - 1 slabs ahead (gemm_mainloop_ring) -
   // for small tiles whose slab of MFMAs is shorter than the memory latency; one workgroup per CU.
   static constexpr int STAGES = STAGES_;
-  static constexpr bool RING = STAGES_ > 2;
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-  static_assert(STAGES_ >= 2 && STAGES_ <= 6 && STAGES_ * (BM_ + BN_) * kRowBytes <= 160 * 1024, "LDS stages");
-  static_assert(STAGES_ == 2 || (DIRECT_ && !B_KMAJOR_ && BM_ <= 128), "ring: direct path of the small tiles");
+  // The 256-row direct tiles take STAGES == 3 to mean: token panel in a ring of three stages, weight panel in two
+  // (gemm_mainloop_fixed16) - exactly the 160 KB of LDS a CU has.
+  static constexpr bool A_RING3 = MFMA16 && STAGES_ == 3;
+  static constexpr bool RING = STAGES_ > 2 && !MFMA16;
+  static constexpr int LDS_BYTES = A_RING3 ? 3 * A_BYTES + 2 * BN * kRowBytes : STAGES * STAGE_BYTES;
+  static_assert(STAGES_ >= 2 && STAGES_ <= 6 && LDS_BYTES <= 160 * 1024, "LDS stages");
+  static_assert(STAGES_ == 2 || A_RING3 || (DIRECT_ && !B_KMAJOR_ && BM_ <= 128), "ring: direct path of the small tiles");
   static_assert(WTM % 32 == 0 && WTN_OUT % 32 == 0, "wave tile must be a multiple of 32x32");
   static_assert(NWAVES % 2 == 0, "lane mapping of the slab layout needs an even wave count");
   static_assert((BM / 16) % NWAVES == 0 && (BN / 16) % NWAVES == 0, "panel rows must split evenly over waves");
@@ -596,10 +599,10 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
 }
 
 // =============================================================================================
-// Direct path of the 256-row tiles: the same two stages of 64-element slabs, accumulated with
-// v_mfma_f32_16x16x32_bf16 in a schedule written out in source order (every MFMA fenced by scheduling
-// barriers), because with one or two wavefronts per SIMD nothing else hides a wait, and an instruction
-// that cannot issue - a load while the address unit's queue is full - holds back the MFMAs behind it.
+// Direct path of the 256-row tiles: 64-element slabs accumulated with v_mfma_f32_16x16x32_bf16 in a schedule
+// written out in source order (every MFMA fenced by scheduling barriers), because with one or two wavefronts
+// per SIMD nothing else hides a wait, and an instruction that cannot issue - a load while the address unit's
+// queue is full - holds back the MFMAs behind it.
 //  * A slab is two K steps of 32.  A step runs its TM x TN MFMAs row group by row group: the token
 //    fragment of a group (16 rows x 32 K) is single-buffered and re-read in place for the next step as
 //    soon as the group's last MFMA has issued (a whole step ahead of its next use); the TN weight
@@ -607,13 +610,20 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
 //  * Two barriers per slab, both in its second step.  The release barrier, behind the step's first four
 //    MFMAs: the stage's last fragment reads were issued at the end of the first step and have returned
 //    (lgkmcnt only), so the stage is free for the slab after next.  The data barrier, behind the first two
-//    row groups: the next slab has landed in the other stage (vmcnt leaves the loads issued since the
-//    release barrier in flight).  One barrier doing both jobs started the loads twelve MFMAs later (1-3 % slower;
-//    the waves run in step, a barrier by itself measures nothing).
+//    row groups: the next slab has landed (vmcnt leaves the loads issued since in flight).  One barrier doing
+//    both jobs started the loads twelve MFMAs later (1-3 % slower; the waves run in step, a barrier by itself
+//    measures nothing).
 //  * The global->LDS loads go out no faster than the address unit takes them, one 1 KB load per wave
-//    behind every fourth or fifth MFMA (16 cycles per load and CU), not in a burst behind the barrier: the
-//    first loads of the slab after next through the rest of the second step, the others during the
-//    first step of the following slab - at least half a slab ahead of the barrier that waits for them.
+//    behind every fourth or fifth MFMA (16 cycles per load and CU), not in a burst behind the barrier.
+//  * Two LDS layouts.  Two stages of (token panel, weight panel): the first loads of the slab after next go
+//    out through the rest of the second step, the others during the first step of the following slab - the
+//    last of them 61 MFMAs ahead of the data barrier that waits for them.  Cfg::A_RING3 (all 160 KB of LDS):
+//    three token stages and two weight stages; the token stage that slab kt + 2 will use was released a slab
+//    ago, so its loads go out during slab kt's first step and only the weight panel's wait for the release
+//    barrier - every load is at least 100 MFMAs ahead of its data barrier.  Cycle stamps around the barriers
+//    (s_memtime, one lane per workgroup) put the data barrier of the two-stage form at 120 cycles per slab on
+//    the SwiGLU GEMM (K = 4096) and at 270 of 2 700 on the down projection (K = 14336), whose panels miss L2
+//    more often; the ring takes the down projection from 2.66 to 2.55 ms and leaves the SwiGLU GEMM where it was.
 // =============================================================================================
 template <class Cfg>
 __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
@@ -627,18 +637,22 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
   constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
   constexpr int L = NJA + NJB;
-  constexpr int STAGE = Cfg::STAGE_BYTES, A_BYTES = Cfg::A_BYTES;
+  constexpr int A_BYTES = Cfg::A_BYTES, B_BYTES = Cfg::BN * kRowBytes;
   constexpr int NM = TM * TN;
   constexpr int BAR = 2 * TN;            // MFMAs of a slab's second step ahead of the data barrier (two row groups)
   constexpr int RPOS = 4;                // ... ahead of the release barrier
+  // Token panel in a ring of three stages: slab kt's token rows sit in stage kt % 3, its weight rows in stage kt % 2.
+  constexpr bool R3 = Cfg::A_RING3;
   // One load per wave behind every LEV-th MFMA.  One per four MFMAs is the address unit's own rate (16 cycles per
   // load and CU).  The four-wave tiles measure faster a notch slower (SwiGLU tile 3 %, down projection 2.4 %, the
   // gathered single-weight GEMM the same either way), the eight-wave tile 1-4 % slower; six is no better than five.
   constexpr int LEV = NWAVES == 4 ? 5 : 4;
-  constexpr int L1 = (NM - RPOS) / LEV < L ? (NM - RPOS) / LEV : L;  // loads of the slab after next that go out in the second step
+  // Two-stage form: loads of the slab after next that go out in the second step (the rest follow in the next slab's first).
+  constexpr int L1 = R3 ? NJB : ((NM - RPOS) / LEV < L ? (NM - RPOS) / LEV : L);
   constexpr int NPRE = (BAR - RPOS) / LEV;  // ... of them ahead of the data barrier (a load follows the last MFMA of its group of LEV)
   static_assert(RPOS >= 0 && RPOS < BAR && NPRE <= L1, "release barrier ahead of the data barrier");
   static_assert(TM >= 3 && TM >= TN && L1 >= 1 && L1 <= L && (L - L1) * LEV <= NM, "schedule does not fit this wave tile");
+  static_assert(!R3 || (NJA * LEV <= NM && RPOS + NJB * LEV <= NM), "ring schedule does not fit this wave tile");
   const int wave = tl.wave_s;
 
   auto wave_uniform = [](const uint16_t* p) {
@@ -654,6 +668,10 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
 #pragma unroll
   for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
 
+  // LDS layout.  Two stages: stage s holds a slab's token panel, then its weight panel.  Ring: three token panels,
+  // then two weight panels.  Token stages are named by their byte offset (a run-time value in the ring form).
+  auto a_stage = [](int s) { return R3 ? s * A_BYTES : s * Cfg::STAGE_BYTES; };
+  auto b_stage = [](int t) { return R3 ? 3 * A_BYTES + t * B_BYTES : t * Cfg::STAGE_BYTES + A_BYTES; };
   // Fragment of K step s: tile row lr, logical 16-byte chunks 4 s + lh (lh = 0..3: 8 K elements each).
   uint32_t koff[2];
 #pragma unroll
@@ -661,27 +679,30 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   const uint32_t a_base = (uint32_t)(tl.wm * Cfg::WTM) * kRowBytes;
   uint32_t b_base[TN];
 #pragma unroll
-  for (int tn = 0; tn < TN; ++tn) b_base[tn] = A_BYTES + (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
+  for (int tn = 0; tn < TN; ++tn) b_base[tn] = (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
 
   zero_acc<Cfg>(acc);
   const int nk = k_len / kBK;
 
   bf16x8_t fa[TM], fb[2][TN];
-  auto read_a = [&](int i, int stage, int ks) {
-    fa[i] = *reinterpret_cast<const bf16x8_t*>(lds + stage * STAGE + a_base + i * 16 * kRowBytes + koff[ks]);
+  auto read_a = [&](int i, int a_off, int ks) {
+    fa[i] = *reinterpret_cast<const bf16x8_t*>(lds + a_off + a_base + i * 16 * kRowBytes + koff[ks]);
   };
-  auto read_b = [&](int buf, int j, int stage, int ks) {
-    fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(lds + stage * STAGE + b_base[j] + koff[ks]);
+  auto read_b = [&](int buf, int j, int b_off, int ks) {
+    fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(lds + b_off + b_base[j] + koff[ks]);
   };
-  // Load l of a slab: the weight panel's first, then the token panel's.
-  auto load = [&](int l, int stage, int kt) {
-    uint8_t* st = lds + stage * STAGE;
-    const int ko = kt * kRowBytes;
-    if (l < NJB)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
-    else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l - NJB], FFNK_LDS_PTR(st + ((l - NJB) * NWAVES + wave) * 1024), 16,
-                                               offA[l - NJB], ko, 0, Cfg::AUX_A);
+  auto load_b = [&](int l, int b_off, int kt) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(lds + b_off + (l * NWAVES + wave) * 1024), 16, offB[l],
+                                             kt * kRowBytes, 0, 0);
+  };
+  auto load_a = [&](int l, int a_off, int kt) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l], FFNK_LDS_PTR(lds + a_off + (l * NWAVES + wave) * 1024), 16, offA[l],
+                                             kt * kRowBytes, 0, Cfg::AUX_A);
+  };
+  // Two-stage form: load l of a slab - the weight panel's first, then the token panel's - into stage t.
+  auto load = [&](int l, int t, int kt) {
+    if (l < NJB) load_b(l, b_stage(t), kt);
+    else load_a(l - NJB, a_stage(t), kt);
   };
   // Four-wave tiles hold 256 accumulator registers per lane, which only fit the accumulation half of the
   // register file.  Left to the builtin, the compiler keeps part of them in ordinary registers and moves
@@ -695,34 +716,38 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
     else
       acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[buf][j], fa[i], acc[i][j], 0, 0, 0);
   };
-  // First K step of slab kt (stage u): behind its MFMAs the fragments of the second step, and the last
-  // loads of slab kt + 1.
+  // First K step of slab kt (weight stage u, token stage at a_cur): behind its MFMAs the fragments of the second
+  // step, and loads: the last ones of slab kt + 1 (two-stage form), or the token panel of slab kt + 2 into the ring
+  // stage at a_ld.
   // The waves leave every barrier together and run the same instructions, so a fragment read that follows the same
   // MFMA in all of them is four 1 KB requests at once against an LDS that moves 128 bytes per cycle
   // (SQ_LDS_CMD_FIFO_FULL counted the waves stalled at issue): the reads are spread over the whole step instead of
   // following the step's first MFMAs in a row (+0.5 %).  Giving each wave its own load slot within a group of LEV
   // MFMAs (one copy of the loop per wave) or holding wave w back by 16 w cycles behind the barrier measured -0.4 %
   // and -3 %: the address unit's FIFO is not filled by the waves' coincidence.
-  auto step0 = [&](int u, int kt, bool next, auto slot) {
+  auto step0 = [&](int u, int a_cur, int a_ld, int kt, bool next, bool next2) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
       mfma(0, m);
       __builtin_amdgcn_sched_barrier(0);
-      if (m % TN == TN / 2 - 1 && m / TN < TN) read_b(1, m / TN, u, 1);   // one per row group
-      if (m % TN == TN - 1) read_a(m / TN, u, 1);
-      if (L1 + m / LEV < L && next) {
-        if (m % LEV == decltype(slot)::value) load(L1 + m / LEV, u ^ 1, kt + 1);
+      if (m % TN == TN / 2 - 1 && m / TN < TN) read_b(1, m / TN, b_stage(u), 1);   // one per row group
+      if (m % TN == TN - 1) read_a(m / TN, a_cur, 1);
+      if constexpr (R3) {
+        if (m % LEV == LEV - 1 && m / LEV < NJA && next2) load_a(m / LEV, a_ld, kt + 2);
+      } else {
+        if (L1 + m / LEV < L && m % LEV == LEV - 1 && next) load(L1 + m / LEV, u ^ 1, kt + 1);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // Second K step: two row groups, the barrier, then behind the MFMAs the first-step fragments of slab
-  // kt + 1 (other stage) and the first loads of slab kt + 2 into this stage.
-  auto step1 = [&](int u, int kt, bool next, bool next2, auto slot) {
+  // Second K step: two row groups, the barriers, then behind the MFMAs the first-step fragments of slab kt + 1
+  // (weight stage u ^ 1, token stage at a_nxt) and loads of slab kt + 2 into the stage the release barrier freed:
+  // its first L1 loads (two-stage form) or its weight panel (ring form).
+  auto step1 = [&](int u, int a_nxt, int kt, bool next, bool next2) {
     __builtin_amdgcn_sched_barrier(0);
-    // Behind the barrier: the first-step fragments of slab kt + 1 (other stage).  Token fragments of the row groups
-    // that ran ahead of the barrier first, then one weight fragment every BSTEP MFMAs (the last one lands a dozen
+    // Behind the barrier: the first-step fragments of slab kt + 1.  Token fragments of the row groups that ran
+    // ahead of the barrier first, then one weight fragment every BSTEP MFMAs (the last one lands a dozen
     // MFMAs before its first use), token fragments of the other groups as their last MFMA issues.
     constexpr int G0 = BAR / TN;                        // row groups ahead of the barrier
     constexpr int BSTEP = (NM - BAR - 2 * G0 - 2) / TN; // spacing of the weight-fragment reads
@@ -734,55 +759,84 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
         __builtin_amdgcn_sched_barrier(0);
       }
       if (m == BAR) {
-        if (next2) dma_wait_barrier<NPRE>();  // slab kt + 1 has landed; the loads of slab kt + 2 issued since stay in flight
+        // slab kt + 1 has landed; the loads of slab kt + 2 issued since stay in flight
+        if (next2) dma_wait_barrier<(R3 ? NJA : 0) + NPRE>();
         else dma_wait_barrier<0>();
         __builtin_amdgcn_sched_barrier(0);
       }
       mfma(1, m);
       __builtin_amdgcn_sched_barrier(0);
       if (next) {
-        if (m >= BAR && m < BAR + 2 * G0 && (m - BAR) % 2 == 0) read_a((m - BAR) / 2, u ^ 1, 0);
+        if (m >= BAR && m < BAR + 2 * G0 && (m - BAR) % 2 == 0) read_a((m - BAR) / 2, a_nxt, 0);
         if (m >= BAR + 2 * G0 && (m - BAR - 2 * G0) % BSTEP == 0 && (m - BAR - 2 * G0) / BSTEP < TN)
-          read_b(0, (m - BAR - 2 * G0) / BSTEP, u ^ 1, 0);
-        if (m / TN >= G0 && m % TN == TN - 1) read_a(m / TN, u ^ 1, 0);
+          read_b(0, (m - BAR - 2 * G0) / BSTEP, b_stage(u ^ 1), 0);
+        if (m / TN >= G0 && m % TN == TN - 1) read_a(m / TN, a_nxt, 0);
       }
-      if (m >= RPOS && (m - RPOS) / LEV < L1 && next2) {
-        if ((m - RPOS) % LEV == decltype(slot)::value) load((m - RPOS) / LEV, u, kt + 2);
+      if (m >= RPOS && (m - RPOS) % LEV == LEV - 1 && (m - RPOS) / LEV < L1 && next2) {
+        if constexpr (R3) load_b((m - RPOS) / LEV, b_stage(u), kt + 2);
+        else load((m - RPOS) / LEV, u, kt + 2);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // Head of the tile: slab 0 whole and the first loads of slab 1, as the steady schedule leaves them.
+  // Head of the tile: slab 0 whole and, of slab 1, what the steady schedule would have issued by now: all of it in
+  // the ring form, its first L1 loads in the two-stage form.
 #pragma unroll
   for (int l = 0; l < L; ++l) load(l, 0, 0);
   if (nk > 1) {
+    if constexpr (R3) {  // token panel first, as the steady schedule issues them
 #pragma unroll
-    for (int l = 0; l < L1; ++l) load(l, 1, 1);
-    dma_wait_barrier<L1>();
+      for (int l = 0; l < NJA; ++l) load_a(l, a_stage(1), 1);
+#pragma unroll
+      for (int l = 0; l < NJB; ++l) load_b(l, b_stage(1), 1);
+      dma_wait_barrier<L>();
+    } else {
+#pragma unroll
+      for (int l = 0; l < L1; ++l) load(l, 1, 1);
+      dma_wait_barrier<L1>();
+    }
   } else {
     dma_wait_barrier<0>();
   }
 #pragma unroll
-  for (int j = 0; j < TN; ++j) read_b(0, j, 0, 0);
+  for (int j = 0; j < TN; ++j) read_b(0, j, b_stage(0), 0);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) read_a(i, 0, 0);
+  for (int i = 0; i < TM; ++i) read_a(i, a_stage(0), 0);
 
   int k0 = 0;
-  constexpr std::integral_constant<int, LEV - 1> slot{};  // every wave issues its load behind the last MFMA of a group of LEV
-  for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches
-    step0(0, k0, true, slot);
-    step1(0, k0, true, true, slot);
-    step0(1, k0 + 1, true, slot);
-    step1(1, k0 + 1, true, true, slot);
-  }
-  constexpr auto last_slot = slot;
-  for (; k0 < nk; k0 += 2) {
-    step0(0, k0, k0 + 1 < nk, last_slot);
-    step1(0, k0, k0 + 1 < nk, k0 + 2 < nk, last_slot);
-    if (k0 + 1 < nk) {
-      step0(1, k0 + 1, k0 + 2 < nk, last_slot);
-      step1(1, k0 + 1, k0 + 2 < nk, k0 + 3 < nk, last_slot);
+  if constexpr (R3) {
+    // token stages of slabs k0, k0 + 1, k0 + 2 (byte offsets), rotated once per slab
+    int s0 = a_stage(0), s1 = a_stage(1), s2 = a_stage(2);
+    // slab kt with its weight panel in stage u
+    auto slab = [&](int u, int kt, bool next, bool next2) {
+      step0(u, s0, s2, kt, next, next2);
+      step1(u, s1, kt, next, next2);
+      const int t = s0;
+      s0 = s1;
+      s1 = s2;
+      s2 = t;
+    };
+    for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches
+      slab(0, k0, true, true);
+      slab(1, k0 + 1, true, true);
+    }
+    for (; k0 < nk; k0 += 2) {
+      slab(0, k0, k0 + 1 < nk, k0 + 2 < nk);
+      if (k0 + 1 < nk) slab(1, k0 + 1, k0 + 2 < nk, k0 + 3 < nk);
+    }
+  } else {
+    auto slab = [&](int u, int kt, bool next, bool next2) {
+      step0(u, a_stage(u), 0, kt, next, next2);
+      step1(u, a_stage(u ^ 1), kt, next, next2);
+    };
+    for (; k0 + 3 < nk; k0 += 2) {  // every guard inside is true: no branches
+      slab(0, k0, true, true);
+      slab(1, k0 + 1, true, true);
+    }
+    for (; k0 < nk; k0 += 2) {
+      slab(0, k0, k0 + 1 < nk, k0 + 2 < nk);
+      if (k0 + 1 < nk) slab(1, k0 + 1, k0 + 2 < nk, k0 + 3 < nk);
     }
   }
   // The compiler does not see that the asm statements are matrix instructions: give the last of them the

@@ -5,14 +5,21 @@
 
 namespace ffnk {
 
+// LDS stages of the 256x256 single-weight tiles on the direct path: 3 = token panel in a ring of three stages, weight
+// panel in two (gemm_mainloop_fixed16).  Measured on the same box against two stages of both: down projection at
+// M = 32768, K = 14336 -3.5 to -4.2 % (2.66 -> 2.55 ms), at M = 1024 -9 % (159 -> 145 us), at M = 4096 -2.3 %.  The
+// SwiGLU tiles keep two stages: the ring measured between -0.8 % and +1.3 % there over three boxes (a tile's head
+// issues two slabs of loads in one burst, which weighs more on a 64-slab contraction than on a 224-slab one), and
+// so did the weight panel in the ring instead of the token panel.
+constexpr int kBigStagesPlain = 3;
 constexpr int kGroupM = 8;       // M-tiles per L2 super-group in the tile order of the SwiGLU GEMM (4: the same, 16 costs 6 % at d=4096, h=14336)
 constexpr int kGroupMPlain = 4;  // single-weight GEMMs: long contractions make wide token panels, 4 x 8 tiles per XCD round re-read fewer of them (1-2 % at K=14336)
 
 // Plain (single-weight) tiles: BN = output columns.
 template <bool GATHER, bool SCATTER, bool DIRECT>
 struct PlainTiles {
-  using T0 = RoutedGemmCfg<256, 256, 2, 4, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
-  using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
+  using T0 = RoutedGemmCfg<256, 256, 2, 4, false, GATHER, SCATTER, DIRECT, kGroupMPlain, false, DIRECT ? kBigStagesPlain : 2>;
+  using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain, false, DIRECT ? kBigStagesPlain : 2>;
   using T2 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
   using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, DIRECT, kGroupMPlain>;
   // 128x128 behind a ring of four LDS stages (direct path; otherwise the two-stage tile)

@@ -48,6 +48,9 @@ def test_tile_table_entries():
     # the four-wave 256x256 tile exists on the direct path only; a staged shape that would pick it runs eight waves
     long_k = _lib.tile_config(_lib.OP_LINEAR_FWD, 32768, 4096, 4096)
     assert long_k["direct_lds"] == 1 and long_k["block_m"] == 256 and long_k["waves_m"] * long_k["waves_n"] == 4
+    # single-weight 256x256 tiles keep their token panel in a ring of three LDS stages (the weight panel in two)
+    assert long_k["lds_stages"] == 3
+    assert _lib.tile_config(_lib.OP_FFN_DOWN, 32768, 4096, 14336)["lds_stages"] == 3
     staged = _lib.tile_config(_lib.OP_LINEAR_FWD, 32768, 4096 + 8, 4096)
     assert staged["direct_lds"] == 0 and staged["block_m"] == 256 and staged["waves_m"] * staged["waves_n"] == 8
     # M <= 8: dot-product streams, one wavefront per 1024-element K slice, no cross-workgroup split

@@ -739,9 +739,9 @@ def test_ffn_forward_keeps_pre_activations_only_when_a_backward_can_follow(dev, 
     from ffn_kernel_amd import ops
     seen = []
     real = ops.masked_ffn_forward
-    def spy(*args, save_pre=False):
+    def spy(*args, save_pre=False, **kw):
         seen.append(save_pre)
-        return real(*args, save_pre=save_pre)
+        return real(*args, save_pre=save_pre, **kw)
     monkeypatch.setattr(ops, "masked_ffn_forward", spy)
     mask = torch.rand(200, generator=torch.Generator().manual_seed(1)) < 0.5
     w = wl.make_ffn("t", 200, 128, 256, mask, seed=2, w_std=0.05).to(dev)

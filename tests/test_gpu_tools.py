@@ -44,7 +44,7 @@ def test_tuner_emits_a_table_the_library_can_compile(dev, tmp_path, capsys):
     entries = re.findall(r"^\s*\{(-?\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},$", text, re.M)
     assert entries and entries[-1][0] == "-1"
     for op, lo, hi, k, n, tile, splits in entries[:-1]:
-        assert int(op) in (0, 1, 2) and int(lo) <= int(hi) and 0 <= int(tile) <= 4 and 1 <= int(splits) <= 16
+        assert int(op) in (0, 1, 2, 3) and int(lo) <= int(hi) and 0 <= int(tile) <= 4 and 1 <= int(splits) <= 16
     recs = json.loads((tmp_path / "t.json").read_text())
     assert {r["op"] for r in recs} == {"ffn_fwd", "linear_fwd", "linear_bwd"}
     lib = _lib.load()
