@@ -528,8 +528,8 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
       out->block_m = 16 * (int)cdiv64(M, 16);
       out->block_n = stream_tile_rows_per_block((int)M, false);
       out->block_k = 128;
-      out->lds_stages = stream_tile_depth((int)M);
-      out->direct_lds = stream_tile_direct((int)M);
+      out->lds_stages = stream_tile_depth((int)M, false);
+      out->direct_lds = stream_tile_direct((int)M, false);
       out->split_k = linear_stream_splits(M, K, N);
     }
     return FFNK_OK;
@@ -551,8 +551,8 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
       // LDS-transposed streams: block_n weight rows (of each matrix) x 128-element chunks, three in flight
       out->block_n = stream_tile_rows_per_block((int)M, up);
       out->block_k = 128;
-      out->lds_stages = stream_tile_depth((int)M);
-      out->direct_lds = stream_tile_direct((int)M);
+      out->lds_stages = stream_tile_depth((int)M, up);
+      out->direct_lds = stream_tile_direct((int)M, up);
       out->split_k = up ? 1 : down_splits(M, K, N);
     }
     if (use_dot_path(M, K, N)) {

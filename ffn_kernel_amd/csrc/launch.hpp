@@ -113,8 +113,8 @@ hipError_t launch_stream_dot_down(const StreamArgs& a, hipStream_t stream);
 bool stream_tile_ok(int M, int d, int h);
 bool stream_tile_down_ok(int M, int Nrows, int K);  // single-weight projection alone (MaskedLinear forward)
 int stream_tile_rows_per_block(int M, bool dual);
-int stream_tile_depth(int M);
-int stream_tile_direct(int M);  // 1: the token-row slab is filled by direct global->LDS loads
+int stream_tile_depth(int M, bool dual);
+int stream_tile_direct(int M, bool dual);  // 1: the token-row slab is filled by direct global->LDS loads
 int stream_tile_down_splits(int M, int d, int h);
 hipError_t launch_stream_tile_up(const StreamArgs& a, hipStream_t stream);
 hipError_t launch_stream_tile_down(const StreamArgs& a, hipStream_t stream);

@@ -40,7 +40,12 @@ constexpr int kTK = 128;    // K elements per chunk (16 pieces of 16 bytes per r
 // dma: the token-row slab is filled by direct global -> LDS loads (no staging registers, which is
 // what lets the 3- and 4-m-tile shapes run two-wavefront workgroups) instead of through registers.
 struct TileShapeEntry { int waves, depth, dma; };
-constexpr TileShapeEntry kTileShapes[4] = {{2, 4, 0}, {2, 3, 0}, {2, 3, 1}, {2, 3, 1}};
+// One table per projection.  Four wavefronts per up-projection workgroup for three and four m-tiles (half the
+// slab traffic per weight byte, 80 KB of LDS, one round of workgroups instead of 1.75 with both modalities at
+// M = 64) measured 1-2 % slower than two at M = 48 and 64 and the same at M = 32; the tables stay equal.
+constexpr TileShapeEntry kTileShapesUp[4] = {{2, 4, 0}, {2, 3, 0}, {2, 3, 1}, {2, 3, 1}};
+constexpr TileShapeEntry kTileShapesDown[4] = {{2, 4, 0}, {2, 3, 0}, {2, 3, 1}, {2, 3, 1}};
+constexpr const TileShapeEntry& tile_shape(int ntm_max, bool dual) { return dual ? kTileShapesUp[ntm_max - 1] : kTileShapesDown[ntm_max - 1]; }
 constexpr int kTMaxM = 64;
 
 struct TileJob {
@@ -178,6 +183,11 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
   for (int w = 0; w < 2; ++w)
 #pragma unroll
     for (int m = 0; m < NTM; ++m) acc[w][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  // Token rows this lane stores in the epilogue: s_perm lives in the staging tiles' memory, which the first chunk
+  // overwrites (every wavefront passes the prologue's barrier between these reads and that write).
+  int out_row[NTM];
+#pragma unroll
+  for (int m = 0; m < NTM; ++m) out_row[m] = (!DUAL && m * 16 + lrow < t.mg) ? s_perm[t.p0 + m * 16 + lrow] : 0;
 
   // One chunk.  STEADY: every chunk whose loads this iteration would issue exists, so the loads are
   // unconditional and the compiler's load-counter waits are exact; otherwise the loads are guarded,
@@ -294,7 +304,7 @@ __device__ __forceinline__ void tile_rows(const StreamArgs& a, const TileJob& t,
           *reinterpret_cast<float4*>(a.P + ((int64_t)t.split * a.M + (t.p0 + row)) * a.Nrows + n_out) =
               make_float4(o[0], o[1], o[2], o[3]);
         } else {
-          uint16_t* dst = a.out + (int64_t)s_perm[t.p0 + row] * a.ldo + n_out;
+          uint16_t* dst = a.out + (int64_t)out_row[m] * a.ldo + n_out;
           if ((reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
             uint2 v2;
             v2.x = pack2bf(o[0], o[1]);
@@ -330,9 +340,11 @@ template <int NTM_MAX, bool DUAL, int kTWaves, int kTD, bool XDMA>
 __global__ __launch_bounds__(kTWaves * kWave, 2) void stream_tile_kernel(const StreamArgs a) {
   __shared__ u32x4_t xs[(XDMA ? kTD : 2) * NTM_MAX * 256];
   __shared__ u32x4_t wst_all[kTWaves * 512];
-  __shared__ int s_perm[kTMaxM];
-  __shared__ int s_nvis;
-  const int n_vis = route64(a.mask, a.M, s_perm, &s_nvis);
+  // The routing table shares the staging tiles' memory (it is read before the first chunk is staged): with four
+  // wavefronts and a ring of three four-m-tile slabs the arrays above are exactly 80 KB, two workgroups per CU.
+  int* s_perm = reinterpret_cast<int*>(wst_all);
+  int* s_nvis_p = s_perm + kTMaxM;
+  const int n_vis = route64(a.mask, a.M, s_perm, s_nvis_p);
   constexpr int ROWS = DUAL ? 16 * kTWaves : 32 * kTWaves;
   const int row_blocks = a.Nrows / ROWS;
   const int per_grp = row_blocks * a.splits;
@@ -356,11 +368,11 @@ __global__ __launch_bounds__(kTWaves * kWave, 2) void stream_tile_kernel(const S
   else tile_rows<1, DUAL, kTWaves, kTD, XDMA>(a, t, s_perm, xs, wst);
 }
 
-static int tile_waves(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].waves; }
+static const TileShapeEntry& shape_for(int M, bool dual) { return tile_shape(cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16), dual); }
 
-int stream_tile_rows_per_block(int M, bool dual) { return (dual ? 16 : 32) * tile_waves(M); }
-int stream_tile_direct(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].dma; }
-int stream_tile_depth(int M) { return kTileShapes[cdiv(M < 1 ? 1 : M > kTMaxM ? kTMaxM : M, 16) - 1].depth; }
+int stream_tile_rows_per_block(int M, bool dual) { return (dual ? 16 : 32) * shape_for(M, dual).waves; }
+int stream_tile_direct(int M, bool dual) { return shape_for(M, dual).dma; }
+int stream_tile_depth(int M, bool dual) { return shape_for(M, dual).depth; }
 
 constexpr int kTMinChunks = 8;  // >= 2 x the deepest ring: lets the kernels run an unconditional prologue
 
@@ -390,8 +402,8 @@ int stream_tile_down_splits(int M, int d, int h) {
 
 template <int NTM_MAX, bool DUAL>
 static void launch_tile_n(const StreamArgs& a, hipStream_t stream) {
-  constexpr int W = kTileShapes[NTM_MAX - 1].waves, D = kTileShapes[NTM_MAX - 1].depth;
-  constexpr bool X = kTileShapes[NTM_MAX - 1].dma != 0;
+  constexpr int W = tile_shape(NTM_MAX, DUAL).waves, D = tile_shape(NTM_MAX, DUAL).depth;
+  constexpr bool X = tile_shape(NTM_MAX, DUAL).dma != 0;
   const int blocks = 2 * (a.Nrows / ((DUAL ? 16 : 32) * W)) * a.splits;
   hipLaunchKernelGGL((stream_tile_kernel<NTM_MAX, DUAL, W, D, X>), dim3(blocks), dim3(W * kWave), 0, stream, a);
 }

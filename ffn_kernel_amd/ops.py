@@ -133,8 +133,9 @@ class _RouteCache(threading.local):
     """The last partition made on this thread and what it was made from."""
     enabled = True
     key = None
-    storage = None  # keeps the mask's memory alive, so that its address cannot be handed to another tensor
+    mask = None     # keeps the mask's memory alive, so that its address cannot be handed to another tensor
     routing = None
+    last = None     # the partition the last forward on this thread ran with (read back by the autograd functions)
 
 
 _route_cache = _RouteCache()
@@ -146,42 +147,42 @@ def set_route_cache(enabled: bool) -> bool:
     old = _route_cache.enabled
     _route_cache.enabled = bool(enabled)
     if not enabled:
-        _route_cache.key = _route_cache.storage = _route_cache.routing = None
+        _route_cache.key = _route_cache.mask = _route_cache.routing = None
     return old
 
 
-def shared_routing(mask: torch.Tensor, M: int):
-    """The row partition for `mask`, made once and shared by the calls that follow with the same mask: the
-    operations of a transformer layer all route by one mask, and each would otherwise launch its own
-    partition kernel ahead of its GEMM.  The one-entry cache is keyed on the mask's memory (held alive by the
-    entry), its view, its version counter - every in-place write through torch bumps it, so a mask changed in
-    place is partitioned again - and the stream.  Returns None where no partition is shared: decode sizes,
-    the cache switched off, tensors without a version counter, a stream under graph capture (a captured
-    graph must not point at memory this cache may drop later)."""
+def shared_routing(mask: torch.Tensor, M: int, stream: int | None = None):
+    """The row partition for `mask` (contiguous, on a GPU), made once and shared by the calls that follow with
+    the same mask: the operations of a transformer layer all route by one mask, and each would otherwise
+    launch its own partition kernel ahead of its GEMM.  The one-entry cache is keyed on the address of the
+    mask's first element (the entry keeps the tensor, so the memory cannot be handed to another one), the row
+    count, the version counter - every in-place write through torch bumps it, so a mask changed in place is
+    partitioned again - and the stream.  Returns None where no partition is shared: decode sizes, the cache
+    switched off, tensors without a version counter, a stream under graph capture (a captured graph must not
+    point at memory this cache may drop later)."""
     if M < _ROUTED_MIN_ROWS or not _route_cache.enabled:
         return None
-    dev = mask.device
     try:
         version = mask._version
     except RuntimeError:  # inference tensors keep no version counter
         return None
     if torch.cuda.is_current_stream_capturing():
         return None
-    storage = mask.untyped_storage()
-    key = (storage.data_ptr(), mask.storage_offset(), mask.stride(0), M, version, dev.index, _stream_ptr(dev))
+    key = (mask.data_ptr(), M, version, _stream_ptr(mask.device) if stream is None else stream)
     if _route_cache.key == key:
         return _route_cache.routing
     routing = route(mask)
-    _route_cache.key, _route_cache.storage, _route_cache.routing = key, storage, routing
+    _route_cache.key, _route_cache.mask, _route_cache.routing = key, mask, routing
     return routing
 
 
-def _routing_arg(routing, mask: torch.Tensor, M: int):
+def _routing_arg(routing, mask: torch.Tensor, M: int, stream: int):
     """(Routing or None, its ffnk_routing_t* or None) for a call: the caller's, else the shared one."""
     if routing is None:
-        routing = shared_routing(mask, M)
+        routing = shared_routing(mask, M, stream)
     elif routing.M != M or routing.perm.device != mask.device:
         raise ValueError(f"routing is for {routing.M} rows on {routing.perm.device}, the call has {M} on {mask.device}")
+    _route_cache.last = routing
     return routing, (routing.ref() if routing is not None else None)
 
 
@@ -210,12 +211,13 @@ def masked_linear_forward(a: torch.Tensor, b1: torch.Tensor, b2: torch.Tensor, m
         return c
     lib = _lib.load()
     with _on_device(dev):
-        routing, rt = _routing_arg(routing, mask, M)
+        stream = _stream_ptr(dev)
+        routing, rt = _routing_arg(routing, mask, M, stream)
         ws_bytes = _lib.workspace_bytes(_lib.OP_LINEAR_FWD, M, K, N)
         ws = _workspace(ws_bytes, dev)
         rc = lib.ffnk_masked_linear_fwd_routed(a.data_ptr(), a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(),
                                                b2.data_ptr(), sk, sn, mask.data_ptr(), c.data_ptr(), N, M, K, N,
-                                               ws.data_ptr(), ws.numel(), _stream_ptr(dev), rt)
+                                               ws.data_ptr(), ws.numel(), stream, rt)
     _lib.check(rc, "ffnk_masked_linear_fwd")
     return c
 
@@ -247,13 +249,14 @@ def masked_linear_backward(grad: torch.Tensor, a: torch.Tensor, b1: torch.Tensor
         return da, db1, db2
     lib = _lib.load()
     with _on_device(dev):
-        routing, rt = _routing_arg(routing, mask, M)
+        stream = _stream_ptr(dev)
+        routing, rt = _routing_arg(routing, mask, M, stream)
         ws_bytes = _lib.workspace_bytes(_lib.OP_LINEAR_BWD, M, K, N)
         ws = _workspace(ws_bytes, dev)
         rc = lib.ffnk_masked_linear_bwd_routed(grad.data_ptr(), grad.stride(0) if M > 1 else max(N, 1), a.data_ptr(),
                                                a.stride(0) if M > 1 else max(K, 1), b1.data_ptr(), b2.data_ptr(), sk, sn,
                                                mask.data_ptr(), da.data_ptr(), K, db1.data_ptr(), db2.data_ptr(), dsk,
-                                               dsn, M, K, N, ws.data_ptr(), ws.numel(), _stream_ptr(dev), rt)
+                                               dsn, M, K, N, ws.data_ptr(), ws.numel(), stream, rt)
     _lib.check(rc, "ffnk_masked_linear_bwd")
     return da, db1, db2
 
@@ -300,13 +303,14 @@ def masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre: bool = False, 
     if save_pre and h > 0 and lib.ffnk_masked_ffn_can_save(M, d, h) and usk == 1 and dsk == 1:
         pre = torch.empty((M, 2 * h), device=dev, dtype=torch.bfloat16)
     with _on_device(dev):
-        routing, rt = _routing_arg(routing, mask, M)
+        stream = _stream_ptr(dev)
+        routing, rt = _routing_arg(routing, mask, M, stream)
         ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_FWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
         head = (a.data_ptr(), a.stride(0) if M > 1 else max(d, 1), ups[0].data_ptr(), ups[1].data_ptr(),
                 ups[2].data_ptr(), ups[3].data_ptr(), usk, usn, downs[0].data_ptr(), downs[1].data_ptr(), dsk, dsn,
                 mask.data_ptr(), out.data_ptr(), d)
-        tail = (M, d, h, ws.data_ptr(), ws.numel(), _stream_ptr(dev), rt)
+        tail = (M, d, h, ws.data_ptr(), ws.numel(), stream, rt)
         if pre is None:
             rc = lib.ffnk_masked_ffn_fwd_routed(*head, None, 0, *tail)
         else:
@@ -366,13 +370,14 @@ def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None, routing
         else:
             ws_bytes = _lib.workspace_bytes(_lib.OP_FFN_BWD, M, d, h)
         ws = _workspace(ws_bytes, dev)
-        routing, rt = _routing_arg(routing, mask, M)
+        stream = _stream_ptr(dev)
+        routing, rt = _routing_arg(routing, mask, M, stream)
         head = (grad.data_ptr(), grad.stride(0) if M > 1 else d, a.data_ptr(), a.stride(0) if M > 1 else d,
                 ups[0].data_ptr(), ups[1].data_ptr(), ups[2].data_ptr(), ups[3].data_ptr(), usk, usn,
                 downs[0].data_ptr(), downs[1].data_ptr(), dsk, dsn, mask.data_ptr())
         tail = (da.data_ptr(), d, dups[0].data_ptr(), dups[1].data_ptr(), dups[2].data_ptr(), dups[3].data_ptr(),
                 gusk, gusn, ddowns[0].data_ptr(), ddowns[1].data_ptr(), gdsk, gdsn, M, d, h, ws.data_ptr(), ws.numel(),
-                _stream_ptr(dev), rt)
+                stream, rt)
         if pre is None:
             rc = lib.ffnk_masked_ffn_bwd_routed(*head, None, 0, *tail)
         else:
@@ -383,16 +388,6 @@ def masked_ffn_backward(grad, a, w1, w2, w3, u1, u2, u3, mask, pre=None, routing
     dw1, dw3, du1, du3 = dups
     dw2, du2 = ddowns
     return da, dw1, dw2, dw3, du1, du2, du3
-
-
-def _forward_routing(mask):
-    """The shared partition for a well-formed mask (None otherwise: the forward's own checks then report it)."""
-    if isinstance(mask, torch.Tensor) and mask.dtype == torch.bool and mask.dim() == 1 and mask.is_cuda:
-        m = mask if mask.stride(0) == 1 or mask.shape[0] <= 1 else None
-        if m is not None:
-            with _on_device(mask.device):
-                return shared_routing(m, m.shape[0])
-    return None
 
 
 class _GradMode(threading.local):
@@ -410,10 +405,12 @@ class MaskedLinear(Function):
     def forward(ctx, a, b1, b2, mask):
         ctx.save_for_backward(a, mask)
         ctx.b1, ctx.b2 = b1, b2
-        # the partition the forward runs with serves the backward too (autograd refuses a saved mask that
+        _route_cache.last = None
+        out = masked_linear_forward(a, b1, b2, mask)
+        # the partition the forward ran with serves the backward too (autograd refuses a saved mask that
         # was changed in place, so it cannot go stale)
-        ctx.routing = _forward_routing(mask)
-        return masked_linear_forward(a, b1, b2, mask, routing=ctx.routing)
+        ctx.routing = _route_cache.last
+        return out
 
     @staticmethod
     @once_differentiable
@@ -442,11 +439,12 @@ class MaskedFFN(Function):
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, a, w1, w2, w3, u1, u2, u3, mask):
         ctx.weights = (w1, w2, w3, u1, u2, u3)
-        ctx.routing = _forward_routing(mask)
+        _route_cache.last = None
         if _grad_mode.enabled and any(ctx.needs_input_grad):
-            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre=True, routing=ctx.routing)
+            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, save_pre=True)
         else:
-            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask, routing=ctx.routing), None
+            out, pre = masked_ffn_forward(a, w1, w2, w3, u1, u2, u3, mask), None
+        ctx.routing = _route_cache.last
         ctx.has_pre = pre is not None
         if pre is None:
             ctx.save_for_backward(a, mask)
