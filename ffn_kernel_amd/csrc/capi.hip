@@ -401,8 +401,12 @@ int fused_bwd_splits(int64_t M, int64_t K, int64_t N, int plan_splits) {
 // Whether the MaskedLinear backward runs its two GEMMs in one launch, and the split-K factor its
 // weight-gradient GEMM is really launched with.  A measured plan and a forced factor are used as they are
 // (that is what the tuner timed); only a factor the rules guessed goes through the fused launch's own model.
+// The fused launch is one decision: it runs when the weights are readable in place and both GEMMs are on a 128x128
+// tile; the weight-gradient plan (rules, measured plan or forced tile) says which of the two - two LDS stages, or
+// the ring of four - and the dx GEMM follows it.
+bool is_128_tile(int tile) { return tile == TILE_128x128_W4 || tile == TILE_128x128_R4; }
 bool bwd_is_fused(int64_t M, int64_t K, const BwdPlan& p, bool w_kmajor) {
-  return w_kmajor && routed_tile(M, K, false, 0, TUNED_NONE) == TILE_128x128_W4 && p.tc.tile == TILE_128x128_W4;
+  return w_kmajor && is_128_tile(routed_tile(M, K, false, 0, TUNED_NONE)) && is_128_tile(p.tc.tile);
 }
 int bwd_dw_launch_splits(int64_t M, int64_t K, int64_t N, const BwdPlan& p, bool fused) {
   if (!fused || p.tc.tuned || forced_splits() >= 1) return p.tc.splits;
@@ -938,7 +942,7 @@ int ffnk_masked_linear_bwd_routed(const uint16_t* g, int64_t g_stride_m, const u
   const int64_t sc = p.dw_k_contig ? dw_stride_k : dw_stride_n;
   s.splits = bwd_dw_launch_splits(M, K, N, p, fused);
   if (s.splits == 1) { s.out[0] = dWv; s.out[1] = dWt; s.out_sr = sr; s.out_sc = sc; }
-  if (fused) FFNK_HIP(launch_fused_bwd(a, s, stream), "fused dx / dW GEMM");
+  if (fused) FFNK_HIP(launch_fused_bwd(a, s, p.tc.tile == TILE_128x128_R4, stream), "fused dx / dW GEMM");
   else FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
   if (s.splits > 1)
     FFNK_HIP(launch_splitk_reduce(P, s.splits, (int)p.R, (int)p.Cc, dWv, dWt, sr, sc, stream), "dW reduce");

@@ -137,7 +137,7 @@ struct RoutedGemmCfg {
   static constexpr bool RING = STAGES_ > 2 && !MFMA16;
   static constexpr int LDS_BYTES = A_RING3 ? 3 * A_BYTES + 2 * BN * kRowBytes : STAGES * STAGE_BYTES;
   static_assert(STAGES_ >= 2 && STAGES_ <= 6 && LDS_BYTES <= 160 * 1024, "LDS stages");
-  static_assert(STAGES_ == 2 || A_RING3 || (DIRECT_ && !B_KMAJOR_ && BM_ <= 128), "ring: direct path of the small tiles");
+  static_assert(STAGES_ == 2 || A_RING3 || (DIRECT_ && BM_ <= 128), "ring: direct path of the small tiles");
   static_assert(WTM % 32 == 0 && WTN_OUT % 32 == 0, "wave tile must be a multiple of 32x32");
   static_assert(NWAVES % 2 == 0, "lane mapping of the slab layout needs an even wave count");
   static_assert((BM / 16) % NWAVES == 0 && (BN / 16) % NWAVES == 0, "panel rows must split evenly over waves");
@@ -883,14 +883,17 @@ __device__ __forceinline__ void gemm_mainloop_ring(const TileLanes<Cfg>& tl,
                                                    const uint32_t (&offA)[TileLanes<Cfg>::NJA],
                                                    const uint16_t* const (&baseB)[TileLanes<Cfg>::NJB],
                                                    const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
-                                                   uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN]) {
+                                                   uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN],
+                                                   const KMajorB& kb = KMajorB()) {
   static_assert(Cfg::RING && !Cfg::MFMA16, "ring schedule of the small direct tiles");
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN, S = Cfg::STAGES, D = S - 1;
   constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
   constexpr int L = NJA + NJB;
   constexpr int STAGE = Cfg::STAGE_BYTES, A_BYTES = Cfg::A_BYTES;
-  constexpr int NM = TM * TN, ND = TM + TN;
+  constexpr bool KM = Cfg::B_KMAJOR;     // weight panel read in place as [K, N] rows: two transposing reads per fragment
+  constexpr int RB = Cfg::BN * 2;        // ... whose rows are this many bytes
+  constexpr int NM = TM * TN, ND = TM + (KM ? 2 * TN : TN);
   constexpr int LQ = (L + 3) / 4;            // loads per K step (a slab's loads go out over four steps)
   constexpr int RPM = (ND + NM - 1) / NM;    // fragment reads behind each MFMA
   constexpr int LPM = (LQ + NM - 1) / NM;    // loads behind each MFMA
@@ -907,8 +910,27 @@ __device__ __forceinline__ void gemm_mainloop_ring(const TileLanes<Cfg>& tl,
   __amdgpu_buffer_rsrc_t rsA[NJA], rsB[NJB];
 #pragma unroll
   for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseA[j]), 0, 0xffffffff, 0x00020000);
+  if constexpr (!KM) {
 #pragma unroll
-  for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
+    for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
+  }
+  // K-major: one base per weight, uniform over the wave; a slab's offset goes into its resource (see gemm_mainloop_slab_dma).
+  uint64_t kw[2] = {0, 0};
+  if constexpr (KM) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const uint64_t v = reinterpret_cast<uint64_t>(kb.w[q]);
+      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+      const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+      kw[q] = ((uint64_t)hi << 32) | lo;
+    }
+  }
+  auto kmajor_rsrc = [&](int kt) {
+    const int ka = kb.kt_first + kt;
+    const bool second = ka >= kb.kt_switch;
+    const uint64_t base = (second ? kw[1] : kw[0]) + (uint64_t)(uint32_t)(second ? ka - kb.kt_switch : ka) * kb.slab_bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+  };
   uint32_t koff[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) koff[s] = lds_swizzle(tl.lr, 2 * s + tl.lh);
@@ -916,28 +938,72 @@ __device__ __forceinline__ void gemm_mainloop_ring(const TileLanes<Cfg>& tl,
   uint32_t b_base[TN];
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) b_base[tn] = A_BYTES + (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
+  uint32_t kaddr[KM ? S : 1][TN][2];  // K-major: LDS address of this lane's two transposing reads per stage and tile (K step: immediate)
+  if constexpr (KM) {
+    // As in gemm_mainloop_slab_dma: row 8 * lh + (i >> 2) of the slab, columns 16 * (group & 1) + 4 * (i & 3) ... of the tile's 32.
+    const uint32_t i = tl.lane & 15, grp16 = tl.lane >> 4;
+    const uint32_t row = 8 * tl.lh + (i >> 2);
+    const uint32_t key = kmajor_swizzle_key<Cfg::BN>(row);
+    const uint32_t lds_addr = (uint32_t)reinterpret_cast<uintptr_t>(FFNK_LDS_PTR(lds));
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const uint32_t unit = (uint32_t)b_frag_row<Cfg>(tl.wn, tn) / 32;
+      const uint32_t in_stage = A_BYTES + row * RB + ((unit ^ key) << 6) + 32 * (grp16 & 1) + 8 * (i & 3);
+#pragma unroll
+      for (int st = 0; st < S; ++st) {
+        kaddr[st][tn][0] = lds_addr + st * STAGE + in_stage;
+        kaddr[st][tn][1] = kaddr[st][tn][0] + 4 * RB;
+      }
+    }
+  }
 
   zero_acc<Cfg>(acc);
   const int nk = k_len / kBK;
 
   bf16x8_t fa[2][TM], fb[2][TN];
-  auto read_frag = [&](int buf, int stage, int ks, int r) {
+  bf16x4_t fb_lo[2][TN], fb_hi[2][TN];  // K-major: halves of a weight fragment as the two reads deliver them
+  // Fragment read r of K step ks: the weight fragments first (K-major: two reads each), then the token fragments.
+  auto read_frag = [&](int buf, int stage, auto ks_tag, int r) {
+    constexpr int ks = decltype(ks_tag)::value;
     const uint8_t* st = lds + stage * STAGE;
-    if (r < TN) fb[buf][r] = *reinterpret_cast<const bf16x8_t*>(st + b_base[r] + koff[ks]);
-    else fa[buf][r - TN] = *reinterpret_cast<const bf16x8_t*>(st + a_base + (r - TN) * 32 * kRowBytes + koff[ks]);
+    if constexpr (KM) {
+      if (r < 2 * TN) {
+        const bf16x4_t v = lds_read_tr16_b64<16 * ks * RB>(kaddr[stage][r / 2][r & 1]);
+        if (r & 1) fb_hi[buf][r / 2] = v;
+        else fb_lo[buf][r / 2] = v;
+      } else {
+        fa[buf][r - 2 * TN] = *reinterpret_cast<const bf16x8_t*>(st + a_base + (r - 2 * TN) * 32 * kRowBytes + koff[ks]);
+      }
+    } else {
+      if (r < TN) fb[buf][r] = *reinterpret_cast<const bf16x8_t*>(st + b_base[r] + koff[ks]);
+      else fa[buf][r - TN] = *reinterpret_cast<const bf16x8_t*>(st + a_base + (r - TN) * 32 * kRowBytes + koff[ks]);
+    }
+  };
+  // K-major: the transposing reads are asm statements whose results the compiler does not wait for.
+  auto frags_ready = [&](int buf) {
+    if constexpr (KM) {
+      kmajor_wait_frags<TN>(fb_lo[buf], fb_hi[buf]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[buf][j] = __builtin_shufflevector(fb_lo[buf][j], fb_hi[buf][j], 0, 1, 2, 3, 4, 5, 6, 7);
+    }
   };
   auto load = [&](int l, int stage, int kt) {
     uint8_t* st = lds + stage * STAGE;
     const int ko = kt * kRowBytes;
-    if (l < NJB)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
-    else
+    if (l < NJB) {
+      if constexpr (KM)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(kmajor_rsrc(kt), FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l],
+                                                 0, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(st + A_BYTES + (l * NWAVES + wave) * 1024), 16, offB[l], ko, 0, 0);
+    } else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l - NJB], FFNK_LDS_PTR(st + ((l - NJB) * NWAVES + wave) * 1024), 16,
                                                offA[l - NJB], ko, 0, Cfg::AUX_A);
   };
   // One K step: the MFMAs on fragment buffer `cur`; behind them the fragment reads of (stage_next, ks_next)
   // into the other buffer and loads [l0, l0 + LQ) of slab kt_dma into stage_dma.
-  auto step = [&](int cur, int stage_next, int ks_next, bool reads, bool dma, int l0, int stage_dma, int kt_dma) {
+  auto step = [&](int cur, int stage_next, auto ks_next, bool reads, bool dma, int l0, int stage_dma, int kt_dma) {
+    frags_ready(cur);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int q = 0; q < NM; ++q) {
@@ -956,16 +1022,20 @@ __device__ __forceinline__ void gemm_mainloop_ring(const TileLanes<Cfg>& tl,
   auto body = [&](auto stage_tag, int kt, bool steady) {
     constexpr int U = decltype(stage_tag)::value, UN = (U + 1) % S, UP = (U + S - 1) % S;
     const bool far = steady || kt + D < nk;        // slab kt + D exists
-    step(0, U, 1, true, far, LQ, UP, kt + D);
-    step(1, U, 2, true, far, 2 * LQ, UP, kt + D);
-    step(0, U, 3, true, far, 3 * LQ, UP, kt + D);
+    constexpr std::integral_constant<int, 0> k0{};
+    constexpr std::integral_constant<int, 1> k1{};
+    constexpr std::integral_constant<int, 2> k2{};
+    constexpr std::integral_constant<int, 3> k3{};
+    step(0, U, k1, true, far, LQ, UP, kt + D);
+    step(1, U, k2, true, far, 2 * LQ, UP, kt + D);
+    step(0, U, k3, true, far, 3 * LQ, UP, kt + D);
     if (steady) {
       dma_wait_barrier<(S - 2) * L>();
     } else {
       const int last = kt + D < nk ? kt + D : nk - 1;  // last slab issued so far
       dma_wait_barrier_n(last > kt + 1 ? (last - kt - 1) * L : 0);
     }
-    step(1, UN, 0, steady || kt + 1 < nk, steady || kt + S < nk, 0, U, kt + S);
+    step(1, UN, k0, steady || kt + 1 < nk, steady || kt + S < nk, 0, U, kt + S);
   };
 
   // Head of the tile: slabs 0 .. D - 1 whole and the first quarter of slab D, as the steady schedule leaves them.
@@ -984,7 +1054,7 @@ __device__ __forceinline__ void gemm_mainloop_ring(const TileLanes<Cfg>& tl,
   }
   dma_wait_barrier_n(issued - L);  // slab 0 has landed
 #pragma unroll
-  for (int r = 0; r < ND; ++r) read_frag(0, 0, 0, r);
+  for (int r = 0; r < ND; ++r) read_frag(0, 0, std::integral_constant<int, 0>{}, r);
 
   int kt = 0;
   for (; kt + 2 * S - 1 < nk; kt += S) static_for<0, S>([&](auto u) { body(u, kt + decltype(u)::value, true); });
@@ -1005,7 +1075,7 @@ __device__ __forceinline__ void gemm_mainloop_direct(const TileLanes<Cfg>& tl,
                                                      uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN],
                                                      const KMajorB& kb = KMajorB()) {
   if constexpr (Cfg::MFMA16) gemm_mainloop_fixed16<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc);
-  else if constexpr (Cfg::RING) gemm_mainloop_ring<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc);
+  else if constexpr (Cfg::RING) gemm_mainloop_ring<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
   else gemm_mainloop_slab_dma<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
 }
 

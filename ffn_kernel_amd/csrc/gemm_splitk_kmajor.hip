@@ -12,7 +12,7 @@ hipError_t launch_splitk_gemm_kmajor(int tile, const SplitKArgs& g, hipStream_t 
     case TILE_256x256_W4: return launch_grouped_splitk<Tiles::T1>(g, stream);
     case TILE_128x128_W4: return launch_grouped_splitk<Tiles::T2>(g, stream);
     case TILE_SMALL_W4: return launch_grouped_splitk<Tiles::T3>(g, stream);
-    case TILE_128x128_R4: return launch_grouped_splitk<Tiles::T4>(g, stream);
+    case TILE_128x128_R4: return launch_grouped_splitk<Tiles::T2>(g, stream);  // no ring here: the group's last slab is cleared in LDS
     default: return hipErrorInvalidValue;
   }
 }

@@ -33,7 +33,9 @@ struct KMajorTiles {
   using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
   using T2 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
   using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
-  using T4 = T2;  // no ring over K-major weights
+  // 128x128 behind a ring of four LDS stages, for the routed GEMMs (the weight-gradient GEMMs, whose last slab is
+  // ragged and cleared in LDS, stay on the two-stage tile)
+  using T4 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, true, kGroupM, true, 4>;
 };
 
 // SwiGLU tiles: BN = gate rows + up rows held in LDS, i.e. BN / 2 output columns.

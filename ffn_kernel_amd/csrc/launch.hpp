@@ -49,7 +49,8 @@ hipError_t launch_splitk_gemm_kmajor(int tile, const SplitKArgs& g, hipStream_t 
 // The MaskedLinear backward's dx GEMM (K-major weights, as launch_linear_gemm_kmajor on the 128x128 tile)
 // and its weight-gradient GEMM (as launch_splitk_gemm on the 128x128 tile) in ONE launch: weight-gradient
 // workgroups first, dx workgroups behind them.
-hipError_t launch_fused_bwd(const GemmArgs& gx, const SplitKArgs& gw, hipStream_t stream);
+// ring: both on the 128x128 tile behind four LDS stages (one workgroup per CU) instead of two stages (two per CU).
+hipError_t launch_fused_bwd(const GemmArgs& gx, const SplitKArgs& gw, bool ring, hipStream_t stream);
 
 // ---- prep.hip: layout passes around the GEMMs ----
 // dst[r, c] (row-major, ld_dst) = src[r * sr + c * sc] for r < rows, c < cols.

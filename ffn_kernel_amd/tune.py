@@ -7,7 +7,8 @@ The lattice is (tile id) x (split-K factor) per operation, layer shape and M buc
   * MaskedFFN forward: the SwiGLU GEMM's tile, and the down projection's (tile, split-K factor), timed
     per stage with the events of ffnk_masked_ffn_fwd_ev;
   * MaskedLinear forward: (tile, split-K factor) of the routed GEMM, whole call;
-  * MaskedLinear backward: the weight-gradient GEMM's split-K factor, whole call.
+  * MaskedLinear backward: the fused dx / weight-gradient launch's tile (128x128 behind two LDS stages, or behind
+    the ring of four) and the weight-gradient GEMM's split-K factor, whole call.
 Every candidate is forced through ffnk_debug_force_tile / ffnk_debug_force_splits and timed min-of-k;
 the baseline is the library's rules and cost model alone (ffnk_debug_force_tile(-2)).  The host never
 knows how many rows each group holds, and a tile's time jumps where a group's tile count crosses a
@@ -43,7 +44,7 @@ GEN_PATH = Path(__file__).resolve().parent / "csrc" / "tile_table_gen.hpp"
 
 # M buckets [lo, hi]; each is measured at its upper end.  Below 65 rows the FFN runs the streaming kernels.
 BUCKETS = [(65, 128), (129, 256), (257, 512), (513, 1024), (1025, 2048), (2049, 4096), (4097, 8192), (8193, 16384),
-           (16385, 32768)]
+           (16385, 32768), (32769, 65536), (65537, 131072)]  # up to the last key of the reference's tables (bf16_ffn_bwd.json)
 FFN_LAYERS = [(1024, 2048), (2048, 8192), (4096, 14336), (5120, 13824), (8192, 28672)]  # (d, h): cfg2, a mid-size layer, cfg4 / cfg5, two larger LLM layers
 LINEAR_LAYERS = [(1024, 1024), (2048, 2048), (4096, 4096), (8192, 8192)]  # (K, N): cfg1 / cfg3 and LLM-size projections
 
@@ -288,7 +289,8 @@ def tune_linear_bwd(K, N, bucket, trials, dev, margin):
     with _Forced(-2, -1):
         base_cfg = _lib.tile_config(_lib.OP_BWD_DW, hi, K, N)
     slabs = max(1, (lo // 4) // 64)  # every factor must leave whole slabs in the smaller group of the smallest scenario
-    cands = [(s, -2, s, lambda M: True) for s in SPLITS if s <= slabs]
+    # tile -2: the rules' tile with the factor forced; tile 4: both GEMMs of the fused launch behind the ring of four stages
+    cands = [((tile, s), tile, s, lambda M: True) for tile in (-2, 4) for s in SPLITS if s <= slabs]
     base, first, full = _tune_call(lambda inp: (lambda: masked_linear_backward(inp[2], inp[0], Wv.T, Wt.T, inp[1])),
                                    scen, cands, trials, margin)
     return {"op": "linear_bwd", "K": K, "N": N, "m_lo": lo, "m_hi": hi, "rules": base_cfg, "rules_ms": base,
@@ -312,9 +314,11 @@ def plans_from(records, margin):
             if key is not None:
                 out.append((TUNED_PLAIN, r["m_lo"], r["m_hi"], r["K"], r["N"], key[0], key[1]))
         elif r["op"] == "linear_bwd":
-            s, _ = _select(r["rules_ms"], r["ms"], margin)
-            if s is not None:
-                tile = {(256, 256): 0, (128, 128): 2}.get((r["rules"]["block_m"], r["rules"]["block_n"]), 2)
+            key, _ = _select(r["rules_ms"], r["ms"], margin)
+            if key is not None:
+                tile, s = key
+                if tile < 0:
+                    tile = {(256, 256): 0, (128, 128): 2}.get((r["rules"]["block_m"], r["rules"]["block_n"]), 2)
                 out.append((TUNED_SPLITK, r["m_lo"], r["m_hi"], r["N"], r["K"], tile, s))  # R = N, Cc = K (dW stored [N, K])
     # one entry per key (the operation is part of it: a linear layer and an FFN's down projection of the
     # same extents are different kernels and keep their own plans)
@@ -401,7 +405,7 @@ def main(argv=None) -> int:
             r = tune_linear_bwd(K, N, b, args.trials, dev, args.margin)
             records.append(r)
             print(f"linear_bwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} (splits {r['rules']['split_k']}) | "
-                  f"splits:ratio {ratios(r['rules_ms'], r['ms'])}", flush=True)
+                  f"(tile, splits):ratio {ratios(r['rules_ms'], r['ms'])}", flush=True)
     plans = plans_from(records, args.margin)
     print(f"{len(plans)} measured plans lose on no scenario and beat the rules by more than {args.margin:.0%}:")
     for e in plans:
