@@ -117,7 +117,8 @@ struct RoutedGemmCfg {
   // Cache policy of the token panel's global->LDS loads.  The down projection's token rows (the routed intermediate,
   // read in place) pass each XCD once: a round of tiles reads a line and no later round does.  Loaded with the
   // non-temporal hint they do not push the weight panels out of L2 (cfg4 down projection 2.91 -> 2.85 ms, M = 16384
-  // 1.47 -> 1.45 ms; no measurable difference on the smaller tiles, which keep the default).  Gathered token rows
+  // 1.47 -> 1.45 ms on the two-stage form; no difference left behind the three-stage token ring, and none on the
+  // smaller tiles, which keep the default).  Gathered token rows
   // are read again by the next rounds (the hint costs 9 % there), and so are the weights (2-4 %).
   static constexpr int AUX_A = (MFMA16 && !GATHER_A_ && SCATTER_C_) ? 2 : 0;
   static constexpr int MT = MFMA16 ? 16 : 32;              // edge of an accumulator tile
