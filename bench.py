@@ -198,7 +198,7 @@ def _bench_linear(args, dev) -> dict:
         step = lambda: masked_linear_backward(w.grad, w.x, w.Wv.T, w.Wt.T, w.mask)
         flops = w_cpu.routed_flops_bwd
         metric = "MaskedLinear bwd routed bf16 TFLOP/s"
-        kernels = "all launches of one backward call (row partition, gather/transpose, fused dx | dW GEMM)"
+        kernels = "all launches of one backward call (row partition unless shared, fused dx | dW GEMM on g and x in place, reduce of the split partials)"
         tile = {"dx": _lib.tile_config(_lib.OP_BWD_DX, M, K, N), "dw": _lib.tile_config(_lib.OP_BWD_DW, M, K, N)}
     else:
         step = lambda: MaskedLinear.apply(w.x, w.Wv.T, w.Wt.T, w.mask)

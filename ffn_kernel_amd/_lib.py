@@ -21,6 +21,7 @@ _SIGNATURES = {
     "ffnk_last_error": (c_char_p, []),
     "ffnk_debug_force_tile": (c_int, [c_int]),
     "ffnk_debug_force_splits": (c_int, [c_int]),
+    "ffnk_debug_force_bwd_gather": (c_int, [c_int]),
     "ffnk_route": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "ffnk_workspace_bytes": (c_size_t, [c_int, c_int64, c_int64, c_int64]),
     "ffnk_workspace_bytes_ffn_bwd": (c_size_t, [c_int64] * 9),
@@ -90,7 +91,7 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 class TileConfig(ctypes.Structure):
     """Mirror of ffnk_tile_config_t."""
     _fields_ = [(n, c_int32) for n in ("path", "block_m", "block_n", "block_k", "waves_m", "waves_n",
-                                       "lds_stages", "group_m", "split_k", "direct_lds")]
+                                       "lds_stages", "group_m", "split_k", "direct_lds", "in_place")]
 
     def as_dict(self) -> dict:
         return {n: getattr(self, n) for n, _ in self._fields_}

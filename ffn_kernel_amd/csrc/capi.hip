@@ -73,6 +73,7 @@ RouteWs carve_route(uint8_t* ws, int64_t M) {
 // Tuner overrides, see ffnk_debug_force_tile / ffnk_debug_force_splits.
 std::atomic<int> g_force_tile{-1};    // 0..3: that tile; -1: table, then rules; -2: rules only
 std::atomic<int> g_force_splits{-1};  // >= 1: that split-K factor where a GEMM can be split
+std::atomic<int> g_force_bwd_gather{-1};  // MaskedLinear backward: 1 = weight gradients from g and x in place, 0 = from transposes, -1 = plan
 
 int forced_tile() {
   const int t = g_force_tile.load(std::memory_order_relaxed);
@@ -106,10 +107,14 @@ int resolve_routing(const ffnk_routing_t* rt, const RouteWs& r, const uint8_t* m
   return FFNK_OK;
 }
 
+// Pseudo tile id of a measured weight-gradient plan: g and x read where they lie (gemm_dw_gather.hpp) on the 128x128 tile.
+constexpr int kTileGatherDw = 5;
+
 struct BwdPlan {
   bool dw_k_contig;  // dW memory is [N, K] (k contiguous): R = N, Cc = K
   int64_t R, Cc;
   TileChoice tc;
+  bool gather;       // weight gradients from g and x in place, where the call's operands allow it (gather_dw_ok)
   int64_t ldt;       // row stride of the transposed operands
   size_t off_wt, off_gt, off_xt, off_p, total;
 };
@@ -119,7 +124,19 @@ BwdPlan plan_bwd(int64_t M, int64_t K, int64_t N, bool dw_k_contig) {
   p.R = dw_k_contig ? N : K;
   p.Cc = dw_k_contig ? K : N;
   p.tc = pick_splitk_tile(M, p.R, p.Cc, use_tuned());
-  if (forced_tile() >= 0) p.tc.tile = forced_tile();
+  // A measured plan names the form (5: in place; 0 / 2 / 4: from transposes).  Where nothing was measured: the in-place
+  // form saves a launch and the transposes' 4 * M * (K + N) bytes of traffic, and its two-stage loop runs the GEMM's
+  // M * K * N products about 15 % slower than the tiles that read transposes; on this part the two balance near
+  // K * N / (K + N) = 1600 (K = N: faster by 19 % at 1024, 15 % at 2048, slower by 9 % at 4096).
+  // Up to 1024 rows the transposes are a launch that moves next to nothing, and the in-place form wins at every size
+  // (by 4-8 % at K = N = 4096, 8-33 % at 8192).
+  p.gather = p.tc.tuned ? p.tc.tile == kTileGatherDw : (K * N <= 1536 * (K + N) || M <= 1024);
+  if (p.tc.tile == kTileGatherDw) p.tc.tile = TILE_128x128_W4;
+  if (forced_tile() >= 0) {
+    p.tc.tile = forced_tile();
+    p.gather = false;
+  }
+  if (const int fg = g_force_bwd_gather.load(std::memory_order_relaxed); fg >= 0) p.gather = fg == 1;
   if (forced_splits() >= 1) p.tc.splits = forced_splits();
   p.ldt = padded_rows(M);
   size_t o = route_ws_bytes(M);
@@ -153,6 +170,7 @@ constexpr FfnBwdPaths kFfnBwdWorstCase{};
 // Weight-gradient split of the in-place path (H, dt1, dt3 read where they lie).
 TileChoice ffn_bwd_in_place_choice(int64_t M, int64_t d, int64_t h) {
   TileChoice tc = pick_splitk_tile(M, h, d, use_tuned());
+  if (tc.tile == kTileGatherDw) tc.tile = TILE_128x128_W4;  // a MaskedLinear plan of the same extents: the form does not exist here
   if (forced_splits() >= 1) tc.splits = forced_splits();
   return tc;
 }
@@ -371,9 +389,11 @@ size_t tiled_down_partial_bytes(int64_t M, int64_t d, int64_t h) {
 // Split-K factor of the weight-gradient GEMM when it shares a launch with the dx GEMM (both on 128x128
 // tiles, two workgroups per CU).  The weight-gradient workgroups are few and long, the dx workgroups many
 // and short and fill the CUs the others leave: the launch lasts as long as the longer of the two, in
-// 64-row slabs of 0.8 us (a 128x128 tile's slab behind two LDS stages waits on its loads: measured).  Unsplit (no partials, no reduce pass, one launch fewer) unless cutting the
-// contraction shortens the estimate by more than 40 % (at M = 8192, K = N = 1024 two ranges measure 7 % slower than one); never more ranges than the plan sized
-// the partials for.
+// 64-row slabs of 0.8 us (a 128x128 tile's slab behind two LDS stages waits on its loads: measured).  Unsplit (no
+// partials, no reduce pass, one launch fewer) unless cutting the contraction shortens the estimate by more than 35 %
+// (K = N = 1024: at M = 8192, estimate 0.75, two or three ranges measure between 7 % slower and 16 % faster than one
+// depending on the mask; at M = 16384, estimate 0.63, 17-26 % faster); never more ranges than the plan sized the
+// partials for.
 int fused_bwd_splits(int64_t M, int64_t K, int64_t N, int plan_splits) {
   const double slots = 2.0 * kCus, t_slab = 0.8;
   const double dw_tiles = 2.0 * (double)cdiv64(N, 128) * (double)cdiv64(K, 128);
@@ -395,7 +415,7 @@ int fused_bwd_splits(int64_t M, int64_t K, int64_t N, int plan_splits) {
       best_t = t;
     }
   }
-  return best_t < 0.6 * unsplit ? best : 1;
+  return best_t < 0.65 * unsplit ? best : 1;
 }
 
 // Whether the MaskedLinear backward runs its two GEMMs in one launch, and the split-K factor its
@@ -405,8 +425,18 @@ int fused_bwd_splits(int64_t M, int64_t K, int64_t N, int plan_splits) {
 // tile; the weight-gradient plan (rules, measured plan or forced tile) says which of the two - two LDS stages, or
 // the ring of four - and the dx GEMM follows it.
 bool is_128_tile(int tile) { return tile == TILE_128x128_W4 || tile == TILE_128x128_R4; }
-bool bwd_is_fused(int64_t M, int64_t K, const BwdPlan& p, bool w_kmajor) {
-  return w_kmajor && is_128_tile(routed_tile(M, K, false, 0, TUNED_NONE)) && is_128_tile(p.tc.tile);
+// The in-place weight-gradient GEMM addresses token rows with 32-bit byte offsets and moves 8-column chunks.
+// (16-byte aligned in memory, so row strides are multiples of 8 as well).
+bool gather_dw_ok(int64_t M, int64_t K, int64_t N, const void* g, int64_t g_stride_m, const void* x, int64_t x_stride_m) {
+  constexpr int64_t k4g = (int64_t)1 << 32;
+  return M > 0 && K >= 8 && N >= 8 && K % 8 == 0 && N % 8 == 0 && g_stride_m % 8 == 0 && x_stride_m % 8 == 0 &&
+         M * g_stride_m * 2 + 2 * N < k4g && M * x_stride_m * 2 + 2 * K < k4g &&
+         ((reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(x)) & 15) == 0;
+}
+// One launch for both GEMMs: the dx GEMM on a 128x128 tile over weights read in place, and the weight gradients on the
+// same tile (the in-place form has no other).
+bool bwd_is_fused(int64_t M, int64_t K, const BwdPlan& p, bool w_kmajor, bool in_place) {
+  return w_kmajor && is_128_tile(routed_tile(M, K, false, 0, TUNED_NONE)) && (in_place || is_128_tile(p.tc.tile));
 }
 int bwd_dw_launch_splits(int64_t M, int64_t K, int64_t N, const BwdPlan& p, bool fused) {
   if (!fused || p.tc.tuned || forced_splits() >= 1) return p.tc.splits;
@@ -422,6 +452,8 @@ int ffnk_version(void) { return FFNK_VERSION; }
 int ffnk_debug_force_tile(int tile) {
   return g_force_tile.exchange(((tile >= 0 && tile < TILE_COUNT) || tile == -2) ? tile : -1);
 }
+
+int ffnk_debug_force_bwd_gather(int on) { return g_force_bwd_gather.exchange((on == 0 || on == 1) ? on : -1); }
 
 int ffnk_debug_force_splits(int splits) { return g_force_splits.exchange((splits >= 1 && splits <= 16) ? splits : -1); }
 
@@ -484,6 +516,7 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   bool dual = false;
   int64_t contraction;
   int splits = 1;
+  bool in_place = false;
   switch (op) {
     case FFNK_OP_LINEAR_FWD: { const RoutedPlan lp = linear_plan(M, K, N); tile = lp.tile; splits = lp.splits; contraction = K; break; }
     case FFNK_OP_FFN_FWD:
@@ -495,8 +528,9 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
       // As launched for the reference's layout (nn.Linear.weight.T views, contiguous g): weights read in place.
       const BwdPlan bp = plan_bwd(M, K, N, true);
       const bool w_kmajor = N > 0 && N % 64 == 0 && K >= 8 && K % 8 == 0 && direct_ok(N, M, N, 8);
-      tile = bp.tc.tile; contraction = M;
-      splits = bwd_dw_launch_splits(M, K, N, bp, bwd_is_fused(M, K, bp, w_kmajor));
+      in_place = bp.gather && gather_dw_ok(M, K, N, nullptr, N, nullptr, K);
+      tile = in_place ? TILE_128x128_W4 : bp.tc.tile; contraction = M;
+      splits = bwd_dw_launch_splits(M, K, N, bp, bwd_is_fused(M, K, bp, w_kmajor, in_place));
       break;
     }
     default: return fail(FFNK_E_OP, "unknown op %d", op);
@@ -513,7 +547,8 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->waves_n = gm.waves_n;
   out->group_m = dual ? 8 : 4;
   out->split_k = splits;
-  out->direct_lds = direct ? 1 : 0;
+  out->direct_lds = (direct || in_place) ? 1 : 0;
+  out->in_place = in_place ? 1 : 0;
   // 4: ring of four stages (128x128); 3: token panel in three stages, weight panel in two (single-weight 256x256 tiles)
   out->lds_stages = !out->direct_lds ? 2 : tile == TILE_128x128_R4 ? 4 : (is_big_tile(tile) && !dual) ? 3 : 2;
   if (op == FFNK_OP_FFN_DOWN && !stream) out->split_k = tiled_down_splits(M, K, N);
@@ -921,29 +956,42 @@ int ffnk_masked_linear_bwd_routed(const uint16_t* g, int64_t g_stride_m, const u
   const int dx_tile = routed_tile(M, K, false, 0, TUNED_NONE);
   // Both GEMMs on the 128x128 tile and the weights readable in place: one launch runs the two side by
   // side (after the transposes it depends on), see below.
-  const bool fused = bwd_is_fused(M, K, p, w_kmajor);
+  const bool gather = p.gather && gather_dw_ok(M, K, N, g, g_stride_m, x, x_stride_m);
+  const bool fused = bwd_is_fused(M, K, p, w_kmajor, gather);
   if (!fused) {
     if (w_kmajor) FFNK_HIP(launch_linear_gemm_kmajor(dx_tile, a, stream), "dx GEMM");
     else FFNK_HIP(launch_linear_gemm(dx_tile, direct_ok(N, M, g_stride_m, ldw), a, stream), "dx GEMM");
   }
 
   // ---- dW_g = x_g^T g_g, contraction over the rows of group g ----
-  uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]
-  uint16_t* XT = reinterpret_cast<uint16_t*>(wsb + p.off_xt);  // [K, ldt]
   float* P = reinterpret_cast<float*>(wsb + p.off_p);
-  FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)N, GT, x, x_stride_m, (int)K, XT, p.ldt, rt.perm, rt.counts,
-                                    (int)M, stream), "g / x transpose");
   SplitKArgs s;
-  s.A = p.dw_k_contig ? GT : XT; s.lda = p.ldt;
-  s.B = p.dw_k_contig ? XT : GT; s.ldb = p.ldt;
   s.P = P; s.counts = rt.counts; s.M = (int)M;
   s.R = (int)p.R; s.Cc = (int)p.Cc; s.splits = p.tc.splits;
   const int64_t sr = p.dw_k_contig ? dw_stride_n : dw_stride_k;
   const int64_t sc = p.dw_k_contig ? dw_stride_k : dw_stride_n;
   s.splits = bwd_dw_launch_splits(M, K, N, p, fused);
   if (s.splits == 1) { s.out[0] = dWv; s.out[1] = dWt; s.out_sr = sr; s.out_sc = sc; }
-  if (fused) FFNK_HIP(launch_fused_bwd(a, s, p.tc.tile == TILE_128x128_R4, stream), "fused dx / dW GEMM");
-  else FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
+  if (gather) {
+    // g and x read where they lie: the row operand of the output is g when dW's memory is [N, K], x otherwise
+    GatherDwArgs gw;
+    gw.G = p.dw_k_contig ? g : x; gw.ldg = p.dw_k_contig ? g_stride_m : x_stride_m;
+    gw.X = p.dw_k_contig ? x : g; gw.ldx = p.dw_k_contig ? x_stride_m : g_stride_m;
+    gw.perm = rt.perm; gw.counts = rt.counts;
+    s.A = s.B = nullptr; s.lda = s.ldb = 0;
+    gw.s = s;
+    if (fused) FFNK_HIP(launch_fused_bwd_gather(a, gw, stream), "fused dx / dW GEMM");
+    else FFNK_HIP(launch_gathered_dw(gw, stream), "dW GEMM");
+  } else {
+    uint16_t* GT = reinterpret_cast<uint16_t*>(wsb + p.off_gt);  // [N, ldt]
+    uint16_t* XT = reinterpret_cast<uint16_t*>(wsb + p.off_xt);  // [K, ldt]
+    FFNK_HIP(launch_gather_transpose2(g, g_stride_m, (int)N, GT, x, x_stride_m, (int)K, XT, p.ldt, rt.perm, rt.counts,
+                                      (int)M, stream), "g / x transpose");
+    s.A = p.dw_k_contig ? GT : XT; s.lda = p.ldt;
+    s.B = p.dw_k_contig ? XT : GT; s.ldb = p.ldt;
+    if (fused) FFNK_HIP(launch_fused_bwd(a, s, p.tc.tile == TILE_128x128_R4, stream), "fused dx / dW GEMM");
+    else FFNK_HIP(launch_splitk_gemm(p.tc.tile, s, stream), "dW split-K GEMM");
+  }
   if (s.splits > 1)
     FFNK_HIP(launch_splitk_reduce(P, s.splits, (int)p.R, (int)p.Cc, dWv, dWt, sr, sc, stream), "dW reduce");
   return FFNK_OK;

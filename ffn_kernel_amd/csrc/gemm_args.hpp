@@ -70,4 +70,15 @@ struct SplitKArgs {
   int64_t out_sr = 0, out_sc = 0;
 };
 
+// Weight-gradient GEMM of the MaskedLinear backward on the untransposed operands (gemm_dw_gather.hpp):
+//   dW_g[r, c] = sum over the rows m of group g of G[m, r] * X[m, c],   rows found through perm.
+// R % 8 == 0, Cc % 8 == 0, R, Cc >= 8, 16-byte aligned rows, and M * ld * 2 + 2 * cols < 2^32 for both operands.
+struct GatherDwArgs {
+  const uint16_t* G; int64_t ldg;   // [M, R] rows in token order (the upstream gradient)
+  const uint16_t* X; int64_t ldx;   // [M, Cc] rows in token order (the layer's input)
+  const int32_t* perm;              // routed position -> token row
+  const int32_t* counts;
+  SplitKArgs s;                     // R, Cc, splits, M, P / out as for the grouped split-K GEMM (A, B, lda, ldb unused)
+};
+
 }  // namespace ffnk

@@ -1358,6 +1358,58 @@ __global__ __launch_bounds__(Cfg::NT) void routed_gemm_kernel(const GemmArgs g) 
   routed_gemm_body<Cfg>(g, lds, (int)blockIdx.x);
 }
 
+// Store a weight-gradient tile: bf16 with the caller's strides when the contraction was not split, fp32 partials
+// otherwise.  acc[i][j][v]: BM-panel row (= output column c) c0 + wm*WTM + i*MT + lr;
+//                           BN-panel row (= output row r) r0 + wn*WTN + j*MT + acc_col(v, lh).
+template <class Cfg>
+__device__ __forceinline__ void splitk_store(const SplitKArgs& g, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN], int grp, int split,
+                                             int r0, int c0, const TileLanes<Cfg>& rl) {
+  constexpr int TM = Cfg::TM, TN = Cfg::TN;
+  constexpr int MT = Cfg::MT, RUNS = Cfg::ACC_N / 4;
+  if (g.out[0] != nullptr) {
+    // single split: the sums are complete, store bf16 with the caller's strides
+    uint16_t* out = g.out[grp];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int c = c0 + rl.wm * Cfg::WTM + i * MT + (int)rl.lr;
+      if (c >= g.Cc) continue;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int q4 = 0; q4 < RUNS; ++q4) {
+          const int r = r0 + rl.wn * Cfg::WTN_OUT + j * MT + acc_col<Cfg>(4 * q4, (int)rl.lh);
+          uint16_t* dst = out + (int64_t)r * g.out_sr + (int64_t)c * g.out_sc;
+          if (g.out_sr == 1 && r + 3 < g.R && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+            uint2 v2;
+            v2.x = pack2bf(acc[i][j][4 * q4], acc[i][j][4 * q4 + 1]);
+            v2.y = pack2bf(acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]);
+            *reinterpret_cast<uint2*>(dst) = v2;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (r + e < g.R) dst[(int64_t)e * g.out_sr] = f2bf(acc[i][j][4 * q4 + e]);  // out_sc == 1: MT lanes -> 2 MT contiguous bytes
+          }
+        }
+      }
+    }
+    return;
+  }
+  float* P = g.P + ((int64_t)(grp * g.splits + split)) * g.R * g.Cc;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int c = c0 + rl.wm * Cfg::WTM + i * MT + (int)rl.lr;
+    if (c >= g.Cc) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int v = 0; v < Cfg::ACC_N; ++v) {
+        const int r = r0 + rl.wn * Cfg::WTN_OUT + j * MT + acc_col<Cfg>(v, (int)rl.lh);
+        if (r < g.R) P[(int64_t)r * g.Cc + c] = acc[i][j][v];  // MT lanes -> MT consecutive floats
+      }
+    }
+  }
+}
+
 // Grouped split-K GEMM of the weight gradients (operands are padded to 64-element slabs, so
 // the direct path always applies).  With Cfg::B_KMAJOR the operand A is not a padded transpose but
 // the original [rows, R] matrix in routed order (see SplitKArgs).
@@ -1438,51 +1490,7 @@ __device__ __forceinline__ void grouped_splitk_body(const SplitKArgs& g, uint8_t
     zero_acc<Cfg>(acc);  // a split without slabs (e.g. an empty modality) contributes exact zeros
   }
 
-  // acc[i][j][v]: BM-panel row (= output column c) c0 + wm*WTM + i*MT + lr;
-  //               BN-panel row (= output row r) r0 + wn*WTN + j*MT + acc_col(v, lh).
-  constexpr int MT = Cfg::MT, RUNS = Cfg::ACC_N / 4;
-  if (g.out[0] != nullptr) {
-    // single split: the sums are complete, store bf16 with the caller's strides
-    uint16_t* out = g.out[grp];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int c = c0 + rl.wm * Cfg::WTM + i * MT + (int)rl.lr;
-      if (c >= g.Cc) continue;
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-#pragma unroll
-        for (int q4 = 0; q4 < RUNS; ++q4) {
-          const int r = r0 + rl.wn * Cfg::WTN_OUT + j * MT + acc_col<Cfg>(4 * q4, (int)rl.lh);
-          uint16_t* dst = out + (int64_t)r * g.out_sr + (int64_t)c * g.out_sc;
-          if (g.out_sr == 1 && r + 3 < g.R && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
-            uint2 v2;
-            v2.x = pack2bf(acc[i][j][4 * q4], acc[i][j][4 * q4 + 1]);
-            v2.y = pack2bf(acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]);
-            *reinterpret_cast<uint2*>(dst) = v2;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (r + e < g.R) dst[(int64_t)e * g.out_sr] = f2bf(acc[i][j][4 * q4 + e]);  // out_sc == 1: MT lanes -> 2 MT contiguous bytes
-          }
-        }
-      }
-    }
-    return;
-  }
-  float* P = g.P + ((int64_t)(grp * g.splits + split)) * g.R * g.Cc;
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int c = c0 + rl.wm * Cfg::WTM + i * MT + (int)rl.lr;
-    if (c >= g.Cc) continue;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-#pragma unroll
-      for (int v = 0; v < Cfg::ACC_N; ++v) {
-        const int r = r0 + rl.wn * Cfg::WTN_OUT + j * MT + acc_col<Cfg>(v, (int)rl.lh);
-        if (r < g.R) P[(int64_t)r * g.Cc + c] = acc[i][j][v];  // MT lanes -> MT consecutive floats
-      }
-    }
-  }
+  splitk_store<Cfg>(g, acc, grp, split, r0, c0, rl);
 }
 
 template <class Cfg>

@@ -52,6 +52,12 @@ hipError_t launch_splitk_gemm_kmajor(int tile, const SplitKArgs& g, hipStream_t 
 // ring: both on the 128x128 tile behind four LDS stages (one workgroup per CU) instead of two stages (two per CU).
 hipError_t launch_fused_bwd(const GemmArgs& gx, const SplitKArgs& gw, bool ring, hipStream_t stream);
 
+// The weight-gradient GEMM of the MaskedLinear backward on g and x as they lie (no transposes; rows found through
+// perm), alone or in one launch with the dx GEMM on the two-stage 128x128 tile.  hipErrorInvalidValue where the
+// operands do not qualify (see GatherDwArgs).
+hipError_t launch_gathered_dw(const GatherDwArgs& gw, hipStream_t stream);
+hipError_t launch_fused_bwd_gather(const GemmArgs& gx, const GatherDwArgs& gw, hipStream_t stream);
+
 // ---- prep.hip: layout passes around the GEMMs ----
 // dst[r, c] (row-major, ld_dst) = src[r * sr + c * sc] for r < rows, c < cols.
 hipError_t launch_strided_copy2d(const uint16_t* src, int64_t sr, int64_t sc, uint16_t* dst, int64_t ld_dst,

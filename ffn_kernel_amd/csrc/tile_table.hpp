@@ -173,9 +173,11 @@ inline TileChoice pick_splitk_tile(int64_t M, int64_t R, int64_t Cc, bool use_ta
   }
   c.tile = TILE_128x128_W4;
   const int64_t tiles = 2 * cdiv64(R, 128) * cdiv64(Cc, 128);
-  int64_t s = cdiv64(2 * kCus, tiles);            // aim at two workgroups per CU
+  int64_t s = cdiv64(2 * kCus, tiles);            // aim at two workgroups per CU ...
   const int64_t slabs = cdiv64(cdiv64(M, 2), 64);  // 64-row slabs per group at an even split
-  if (s > slabs) s = slabs;
+  // ... with at least 16 slabs to each range: below that the partials and the reduce pass cost more than the idle CUs
+  // (K = N = 1024, M = 256 ... 1024: one range is 20-30 % faster than the two to four that fill the chip)
+  if (s > slabs / 16) s = slabs / 16;
   if (s > 16) s = 16;
   if (s < 1) s = 1;
   c.splits = (int)s;

@@ -7,9 +7,10 @@ The lattice is (tile id) x (split-K factor) per operation, layer shape and M buc
   * MaskedFFN forward: the SwiGLU GEMM's tile, and the down projection's (tile, split-K factor), timed
     per stage with the events of ffnk_masked_ffn_fwd_ev;
   * MaskedLinear forward: (tile, split-K factor) of the routed GEMM, whole call;
-  * MaskedLinear backward: the fused dx / weight-gradient launch's tile (128x128 behind two LDS stages, or behind
-    the ring of four) and the weight-gradient GEMM's split-K factor, whole call.
-Every candidate is forced through ffnk_debug_force_tile / ffnk_debug_force_splits and timed min-of-k;
+  * MaskedLinear backward: the form of the weight-gradient GEMM (from routed transposes on the rules' tile, the same
+    with both GEMMs of the fused launch behind the ring of four LDS stages, or from g and x read in place) and its
+    split-K factor, whole call.
+Every candidate is forced through ffnk_debug_force_tile / ffnk_debug_force_splits (/ ffnk_debug_force_bwd_gather) and timed min-of-k;
 the baseline is the library's rules and cost model alone (ffnk_debug_force_tile(-2)).  The host never
 knows how many rows each group holds, and a tile's time jumps where a group's tile count crosses a
 multiple of the CU count, so one mask says little about a bucket: every bucket is measured on several
@@ -38,6 +39,7 @@ from . import _lib
 from .ops import masked_linear_backward, masked_linear_forward
 
 TILES = {0: "256x256/8w", 1: "256x256/4w", 2: "128x128/4w", 3: "small/4w", 4: "128x128/ring4"}
+TILE_IN_PLACE = 5  # weight-gradient plans only (kTileGatherDw in csrc/capi.hip): g and x read where they lie
 SPLITS = (1, 2, 3, 4, 6, 7, 8, 12, 14, 16)
 TUNED_PLAIN, TUNED_DUAL, TUNED_SPLITK, TUNED_DOWN = 0, 1, 2, 3  # TunedOp in csrc/tile_table.hpp
 GEN_PATH = Path(__file__).resolve().parent / "csrc" / "tile_table_gen.hpp"
@@ -75,20 +77,24 @@ def _randn(shape, std, gen, dev):
 
 
 class _Forced:
-    """Force (tile, splits) for the duration of a block; always back to the table afterwards."""
+    """Force (tile, splits) for the duration of a block; always back to the table afterwards.  The weight-gradient
+    form goes with the tile: TILE_IN_PLACE forces it on (over the rules' tile for the dx GEMM), any other candidate
+    forces it off, and the baseline (-2, -1) leaves it to the rules."""
 
     def __init__(self, tile, splits):
         self.tile, self.splits = tile, splits
 
     def __enter__(self):
         lib = _lib.load()
-        lib.ffnk_debug_force_tile(self.tile)
+        lib.ffnk_debug_force_tile(-2 if self.tile == TILE_IN_PLACE else self.tile)
         lib.ffnk_debug_force_splits(self.splits)
+        lib.ffnk_debug_force_bwd_gather(-1 if (self.tile, self.splits) == (-2, -1) else int(self.tile == TILE_IN_PLACE))
 
     def __exit__(self, *exc):
         lib = _lib.load()
         lib.ffnk_debug_force_tile(-1)
         lib.ffnk_debug_force_splits(-1)
+        lib.ffnk_debug_force_bwd_gather(-1)
 
 
 def _ffn_stage_ms(x, W, mask, trials, ev):
@@ -288,12 +294,15 @@ def tune_linear_bwd(K, N, bucket, trials, dev, margin):
     scen = [(_randn((M, K), 1.0, gen, dev), mask, _randn((M, N), 1.0, gen, dev)) for M, mask in _scenarios(bucket, gen, dev)]
     with _Forced(-2, -1):
         base_cfg = _lib.tile_config(_lib.OP_BWD_DW, hi, K, N)
+    with _Forced(-2, 1):
+        xpose_cfg = _lib.tile_config(_lib.OP_BWD_DW, hi, K, N)  # the rules' tile for the form that reads transposes
     slabs = max(1, (lo // 4) // 64)  # every factor must leave whole slabs in the smaller group of the smallest scenario
-    # tile -2: the rules' tile with the factor forced; tile 4: both GEMMs of the fused launch behind the ring of four stages
-    cands = [((tile, s), tile, s, lambda M: True) for tile in (-2, 4) for s in SPLITS if s <= slabs]
+    # tile -2: the rules' tile, from transposes, with the factor forced; tile 4: both GEMMs of the fused launch behind
+    # the ring of four stages; TILE_IN_PLACE: no transposes
+    cands = [((tile, s), tile, s, lambda M: True) for tile in (-2, 4, TILE_IN_PLACE) for s in SPLITS if s <= slabs]
     base, first, full = _tune_call(lambda inp: (lambda: masked_linear_backward(inp[2], inp[0], Wv.T, Wt.T, inp[1])),
                                    scen, cands, trials, margin)
-    return {"op": "linear_bwd", "K": K, "N": N, "m_lo": lo, "m_hi": hi, "rules": base_cfg, "rules_ms": base,
+    return {"op": "linear_bwd", "K": K, "N": N, "m_lo": lo, "m_hi": hi, "rules": base_cfg, "rules_xpose": xpose_cfg, "rules_ms": base,
             "first_ms": first, "ms": full}
 
 
@@ -318,7 +327,7 @@ def plans_from(records, margin):
             if key is not None:
                 tile, s = key
                 if tile < 0:
-                    tile = {(256, 256): 0, (128, 128): 2}.get((r["rules"]["block_m"], r["rules"]["block_n"]), 2)
+                    tile = {(256, 256): 0, (128, 128): 2}.get((r["rules_xpose"]["block_m"], r["rules_xpose"]["block_n"]), 2)
                 out.append((TUNED_SPLITK, r["m_lo"], r["m_hi"], r["N"], r["K"], tile, s))  # R = N, Cc = K (dW stored [N, K])
     # one entry per key (the operation is part of it: a linear layer and an FFN's down projection of the
     # same extents are different kernels and keep their own plans)
@@ -340,6 +349,21 @@ def render_header(plans) -> str:
     return "\n".join(lines)
 
 
+def read_header(path) -> list:
+    """The entries of a generated header (the terminator excluded), as render_header wrote them."""
+    import re
+    out = []
+    for m in re.finditer(r"^\s*\{(-?\d+(?:,\s*-?\d+){6})\},", Path(path).read_text(), re.M):
+        e = tuple(int(v) for v in m.group(1).split(","))
+        if e[0] >= 0:
+            out.append(e)
+    return out
+
+
+OPS = ("ffn_fwd", "linear_fwd", "linear_bwd")
+OP_KINDS = {"ffn_fwd": (TUNED_DUAL, TUNED_DOWN), "linear_fwd": (TUNED_PLAIN,), "linear_bwd": (TUNED_SPLITK,)}
+
+
 def _fmt_list(ts):
     return "/".join(f"{t:.3f}" for t in ts)
 
@@ -356,7 +380,12 @@ def main(argv=None) -> int:
                     help="MaskedFFN layer to measure besides the default ones (repeatable)")
     ap.add_argument("--linear", action="append", default=None, metavar="K,N",
                     help="MaskedLinear layer to measure besides the default ones (repeatable)")
+    ap.add_argument("--ops", default=",".join(OPS), help="operations to measure (comma separated); --emit keeps the "
+                    f"plans that {GEN_PATH.name} holds for the others")
     args = ap.parse_args(argv)
+    ops = [o for o in args.ops.split(",") if o]
+    if not ops or any(o not in OPS for o in ops):
+        ap.error(f"--ops takes a comma separated subset of {', '.join(OPS)}")
 
     def pairs(specs, default):
         out = list(default)
@@ -385,7 +414,7 @@ def main(argv=None) -> int:
     def ratios(base, cand):
         return "  ".join(f"{k}:" + "/".join(f"{t / b_:.2f}" for t, b_ in zip(ts, base)) for k, ts in cand.items()) or "-"
 
-    for d, h in ffn_layers:
+    for d, h in (ffn_layers if "ffn_fwd" in ops else []):
         for b in buckets:
             if b[1] * h * 2 > 4 << 30:
                 continue
@@ -398,15 +427,23 @@ def main(argv=None) -> int:
                   f" | down (tile, splits):ratio {ratios(r['rules_down_ms'], r['down_ms'])}", flush=True)
     for K, N in linear_layers:
         for b in buckets:
-            r = tune_linear_fwd(K, N, b, args.trials, dev, args.margin)
-            records.append(r)
-            print(f"linear_fwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} | (tile, splits):ratio "
-                  f"{ratios(r['rules_ms'], r['ms'])}", flush=True)
-            r = tune_linear_bwd(K, N, b, args.trials, dev, args.margin)
-            records.append(r)
-            print(f"linear_bwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} (splits {r['rules']['split_k']}) | "
-                  f"(tile, splits):ratio {ratios(r['rules_ms'], r['ms'])}", flush=True)
+            if "linear_fwd" in ops:
+                r = tune_linear_fwd(K, N, b, args.trials, dev, args.margin)
+                records.append(r)
+                print(f"linear_fwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} | (tile, splits):ratio "
+                      f"{ratios(r['rules_ms'], r['ms'])}", flush=True)
+            if "linear_bwd" in ops:
+                r = tune_linear_bwd(K, N, b, args.trials, dev, args.margin)
+                records.append(r)
+                print(f"linear_bwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} (splits {r['rules']['split_k']}"
+                      f"{', in place' if r['rules']['in_place'] else ''}) | (tile, splits):ratio {ratios(r['rules_ms'], r['ms'])}",
+                      flush=True)
     plans = plans_from(records, args.margin)
+    if len(ops) < len(OPS):
+        measured = {k for o in ops for k in OP_KINDS[o]}
+        kept = [e for e in read_header(GEN_PATH) if e[0] not in measured]
+        print(f"{len(kept)} plans of the operations not measured in this run are kept from {GEN_PATH.name}")
+        plans = sorted(plans + kept)
     print(f"{len(plans)} measured plans lose on no scenario and beat the rules by more than {args.margin:.0%}:")
     for e in plans:
         print("   op=%d M in [%d, %d] k=%d n=%d -> tile %d, splits %d" % e)

@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define FFNK_VERSION 101
+#define FFNK_VERSION 102
 
 #if defined(__GNUC__)
 #define FFNK_API __attribute__((visibility("default")))
@@ -77,6 +77,8 @@ typedef struct ffnk_tile_config_t {
   int32_t group_m;     /* M-tiles per L2 super-group in the tile order             */
   int32_t split_k;     /* contraction splits reduced by a second kernel (1 = none) */
   int32_t direct_lds;  /* 1 = global->LDS loads bypass registers                   */
+  int32_t in_place;    /* FFNK_OP_BWD_DW: 1 = the weight-gradient GEMM reads g and x
+                          where they lie, 0 = routed transposes written first      */
 } ffnk_tile_config_t;
 
 FFNK_API int ffnk_version(void);
@@ -139,6 +141,10 @@ FFNK_API int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile
  */
 FFNK_API int ffnk_debug_force_tile(int tile);
 FFNK_API int ffnk_debug_force_splits(int splits);
+/* MaskedLinear backward, tuner-only like the two above: 1 = the weight-gradient GEMM reads g and x where they lie
+ * (rows found through perm) wherever the operands allow it, 0 = it reads routed, padded transposes written by an
+ * elementwise pass first, -1 = the plan decides.  Returns the previous value. */
+FFNK_API int ffnk_debug_force_bwd_gather(int on);
 
 /*
  * MaskedLinear forward — replaces _bf16_linear_forward (ffn_kernel/linear.py:418-452):

@@ -98,16 +98,28 @@ def test_tile_table_entries():
     assert _lib.tile_config(_lib.OP_LINEAR_FWD, 1, 4096, 4096)["path"] == _lib.PATH_STREAM
     assert _lib.tile_config(_lib.OP_LINEAR_FWD, 64, 4096, 4096)["path"] == _lib.PATH_STREAM
     assert _lib.tile_config(_lib.OP_LINEAR_FWD, 64, 4096, 4100)["path"] == _lib.PATH_MFMA_TILED  # ragged N
-    # the factor reported is the one launched: the fused dx / dW launch of the usual layout runs cfg3's
-    # weight-gradient GEMM unsplit, whatever the stand-alone GEMM's rule would pick; a forced factor is kept
-    dw = _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)
-    assert dw["split_k"] == 1
+    # the factor reported is the one launched: by the rules alone, the fused dx / dW launch of the usual layout runs
+    # cfg3's weight-gradient GEMM unsplit and on g and x where they lie, whatever the stand-alone GEMM's rule would
+    # pick; a forced factor and a forced form are kept
     lib = _lib.load()
     try:
+        lib.ffnk_debug_force_tile(-2)
+        dw = _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)
+        assert dw["split_k"] == 1 and dw["in_place"] == 1 and (dw["block_m"], dw["block_n"], dw["lds_stages"]) == (128, 128, 2)
+        big = _lib.tile_config(_lib.OP_BWD_DW, 8192, 4096, 4096)      # compute-bound: routed transposes, 256x256 tiles
+        assert big["in_place"] == 0 and big["block_m"] == 256
+        assert _lib.tile_config(_lib.OP_BWD_DW, 512, 4096, 4096)["in_place"] == 1   # few rows: the transposes are a launch for nothing
+        assert _lib.tile_config(_lib.OP_BWD_DW, 8192, 1028, 1024)["in_place"] == 0  # K % 8 != 0: rows are not 16-byte chunks
         lib.ffnk_debug_force_splits(4)
         assert _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)["split_k"] == 4
+        lib.ffnk_debug_force_bwd_gather(0)
+        assert _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)["in_place"] == 0
+        lib.ffnk_debug_force_bwd_gather(1)
+        assert _lib.tile_config(_lib.OP_BWD_DW, 8192, 4096, 4096)["in_place"] == 1
     finally:
         lib.ffnk_debug_force_splits(-1)
+        lib.ffnk_debug_force_tile(-1)
+        lib.ffnk_debug_force_bwd_gather(-1)
     with pytest.raises(ValueError):
         _lib.tile_config(77, 1, 1, 1)
 
@@ -253,8 +265,12 @@ def test_measured_plans_are_consulted_before_the_rules():
             for M in (hi, (lo + hi) // 2):
                 cfg = _lib.tile_config(_lib.OP_BWD_DW, M, n, k)
                 assert cfg["split_k"] == splits, (op, M, k, n, cfg)
+                # the plan names the form as well: tile 5 reads g and x in place, any other tile reads transposes
+                assert cfg["in_place"] == int(tile == tune.TILE_IN_PLACE), (op, M, k, n, cfg)
                 if tile in geom:
                     assert (cfg["block_m"], cfg["block_n"]) == geom[tile][:2]
+                if tile == tune.TILE_IN_PLACE:
+                    assert (cfg["block_m"], cfg["block_n"], cfg["lds_stages"]) == (128, 128, 2)
             checked += 1
     assert checked > 0 or not entries
     ops_seen = {e[0] for e in entries}

@@ -880,6 +880,94 @@ def test_linear_bwd_fused_launch(dev, M, K, N, p):
         assert torch.equal(a, b)
 
 
+@pytest.fixture
+def force_bwd_form():
+    """ffnk_debug_force_bwd_gather / ffnk_debug_force_splits for one test; back to the plans afterwards."""
+    lib = _lib.load()
+
+    def force(in_place, splits):
+        lib.ffnk_debug_force_bwd_gather(in_place)
+        lib.ffnk_debug_force_splits(splits)
+    try:
+        yield force
+    finally:
+        lib.ffnk_debug_force_bwd_gather(-1)
+        lib.ffnk_debug_force_splits(-1)
+
+
+@pytest.mark.parametrize("splits", [-1, 1, 3])
+@pytest.mark.parametrize("in_place", [0, 1])
+@pytest.mark.parametrize("M,K,N,p,layout", [
+    (37, 48, 40, 0.5, "views"),          # one ragged slab per modality, ragged tiles
+    (300, 128, 136, 0.5, "views"),
+    (1000, 256, 320, 0.3, "kn"),         # weights stored [K, N]: the gradients' memory is [K, N] as well
+    (777, 136, 200, 0.0, "views"),       # no visual rows
+    (515, 128, 128, 1.0, "kn"),          # no text rows
+    (4100, 1024, 384, 0.5, "views"),     # one launch for both GEMMs
+    (2500, 512, 1024, 0.6, "strided"),   # g and x are column slices of wider tensors
+])
+def test_linear_bwd_weight_gradients_in_place_and_from_transposes(dev, force_bwd_form, in_place, splits, M, K, N, p, layout):
+    """The weight-gradient GEMM has two forms - g and x read where they lie (rows found through the partition), or
+    routed transposes written first - and each runs split or unsplit: every combination against the oracle, exact
+    zeros for an absent modality, bit-identical on a second call."""
+    note(f"linear bwd forms in_place={in_place} splits={splits} M={M} K={K} N={N} p={p} {layout}")
+    gen = torch.Generator().manual_seed(M + N + 7)
+    mask = torch.rand(M, generator=gen) < p if 0 < p < 1 else torch.full((M,), bool(p))
+    w = wl.make_linear("t", M, K, N, mask, seed=M + 2, with_grad=True, w_std=0.05)
+    d = w.to(dev)
+    g, x = d.grad, d.x
+    if layout == "strided":
+        gw_, xw_ = torch.full((M, N + 24), float("nan"), device=dev, dtype=torch.bfloat16), torch.full(
+            (M, K + 40), float("nan"), device=dev, dtype=torch.bfloat16)
+        gw_[:, 8:8 + N] = g
+        xw_[:, 16:16 + K] = x
+        g, x = gw_[:, 8:8 + N], xw_[:, 16:16 + K]
+    if layout == "kn":
+        b1, b2 = d.Wv.T.contiguous(), d.Wt.T.contiguous()
+    else:
+        b1, b2 = d.Wv.T, d.Wt.T
+    force_bwd_form(in_place, splits)
+    assert _lib.tile_config(_lib.OP_BWD_DW, M, K, N)["in_place"] == in_place
+    dx, db1, db2 = masked_linear_backward(g, x, b1, b2, d.mask)
+    again = masked_linear_backward(g, x, b1, b2, d.mask)
+    force_bwd_form(-1, -1)
+    torch.cuda.synchronize()
+    assert db1.stride() == b1.stride()
+    rdx, rdWv, rdWt = cref.linear_bwd(w.grad, w.x, w.Wv, w.Wt, w.mask)
+    assert_close(dx, rdx, "dx")
+    assert_close(db1.T, rdWv, "dWv")
+    assert_close(db2.T, rdWt, "dWt")
+    if p == 1.0:
+        assert torch.count_nonzero(db2) == 0
+    if p == 0.0:
+        assert torch.count_nonzero(db1) == 0
+    for a, b in zip((dx, db1, db2), again):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("in_place", [0, 1])
+def test_linear_bwd_non_finite_rows_stay_in_their_modality(dev, force_bwd_form, in_place):
+    """Inf / NaN in the text rows of g and x reach dW_t only: the visual gradient is what it is without them, also
+    where a slab of 64 contraction rows holds the end of one modality (rows past it are cleared, not multiplied by 0)."""
+    note(f"linear bwd non-finite isolation in_place={in_place}")
+    M, K, N = 1000, 256, 192
+    mask = torch.rand(M, generator=torch.Generator().manual_seed(5)) < 0.4
+    w = wl.make_linear("t", M, K, N, mask, seed=9, with_grad=True, w_std=0.05)
+    d = w.to(dev)
+    g, x = d.grad.clone(), d.x.clone()
+    text = (~d.mask).nonzero().flatten()
+    g[text[::3], ::5] = float("inf")
+    x[text[1::3], ::7] = float("nan")
+    x[text[2::3], 1::7] = float("-inf")
+    force_bwd_form(in_place, -1)
+    _, clean_v, _ = masked_linear_backward(d.grad, d.x, d.Wv.T, d.Wt.T, d.mask)
+    dx, dWv, dWt = masked_linear_backward(g, x, d.Wv.T, d.Wt.T, d.mask)
+    force_bwd_form(-1, -1)
+    assert torch.equal(dWv, clean_v)
+    assert torch.isfinite(dx[d.mask]).all()
+    assert not torch.isfinite(dWt).all()
+
+
 @pytest.mark.parametrize("M,d,h,layout", [(300, 256, 512, "views"), (2100, 512, 1024, "views"), (4100, 256, 1024, "views"),
                                           (300, 256, 512, "down_contig"), (333, 72, 200, "views"),
                                           (500, 128, 96, "views")])
