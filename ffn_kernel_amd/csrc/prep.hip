@@ -202,28 +202,49 @@ hipError_t launch_swiglu_bwd(const uint16_t* pre, int64_t ld_pre, uint16_t* T13,
 }
 
 // out_g[r * sr + c * sc] = bf16(P[g][0][r][c] + P[g][1][r][c] + ...), summed in split order so
-// that the result does not depend on scheduling.
+// that the result does not depend on scheduling.  VEC: four consecutive columns per thread (16-byte loads of the
+// partials, one 8-byte store), for outputs whose columns are contiguous (sc == 1) and Cc % 4 == 0.
+template <bool VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ P, int splits, int R, int Cc,
                                                             uint16_t* __restrict__ out0,
                                                             uint16_t* __restrict__ out1, int64_t sr, int64_t sc) {
   const int64_t plane = (int64_t)R * Cc;
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * (VEC ? 4 : 1);
   if (idx >= plane) return;
   const int g = blockIdx.y;
   const float* p = P + (int64_t)g * splits * plane + idx;
-  float s = 0.f;
-  for (int k = 0; k < splits; ++k) s += p[(int64_t)k * plane];
-  const int r = (int)(idx / Cc), c = (int)(idx % Cc);
   uint16_t* out = g == 0 ? out0 : out1;
-  out[(int64_t)r * sr + (int64_t)c * sc] = f2bf(s);
+  const int r = (int)(idx / Cc), c = (int)(idx % Cc);
+  if constexpr (VEC) {
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k = 0; k < splits; ++k) {
+      const float4 v = *reinterpret_cast<const float4*>(p + (int64_t)k * plane);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    uint2 v2;
+    v2.x = pack2bf(s.x, s.y);
+    v2.y = pack2bf(s.z, s.w);
+    *reinterpret_cast<uint2*>(out + (int64_t)r * sr + c) = v2;
+  } else {
+    float s = 0.f;
+    for (int k = 0; k < splits; ++k) s += p[(int64_t)k * plane];
+    out[(int64_t)r * sr + (int64_t)c * sc] = f2bf(s);
+  }
 }
 
 hipError_t launch_splitk_reduce(const float* P, int splits, int R, int Cc, uint16_t* out0, uint16_t* out1,
                                 int64_t sr, int64_t sc, hipStream_t stream) {
   if (R <= 0 || Cc <= 0) return hipSuccess;
   const int64_t plane = (int64_t)R * Cc;
-  dim3 grid((unsigned)cdiv64(plane, 256), 2);
-  hipLaunchKernelGGL(splitk_reduce_kernel, grid, dim3(256), 0, stream, P, splits, R, Cc, out0, out1, sr, sc);
+  const bool vec = sc == 1 && Cc % 4 == 0 && sr % 4 == 0 && ((reinterpret_cast<uintptr_t>(out0) | reinterpret_cast<uintptr_t>(out1)) & 7) == 0 &&
+                   (reinterpret_cast<uintptr_t>(P) & 15) == 0;
+  if (vec) {
+    dim3 grid((unsigned)cdiv64(plane / 4, 256), 2);
+    hipLaunchKernelGGL(splitk_reduce_kernel<true>, grid, dim3(256), 0, stream, P, splits, R, Cc, out0, out1, sr, sc);
+  } else {
+    dim3 grid((unsigned)cdiv64(plane, 256), 2);
+    hipLaunchKernelGGL(splitk_reduce_kernel<false>, grid, dim3(256), 0, stream, P, splits, R, Cc, out0, out1, sr, sc);
+  }
   return hipGetLastError();
 }
 
