@@ -46,7 +46,9 @@ __host__ __device__ constexpr uint32_t lds_swizzle(uint32_t r, uint32_t c) {  //
 // global->LDS loads).  ds_read_b64_tr_b16 turns it into MFMA operands: within a group of 16 lanes,
 // lane j addresses 4 consecutive elements and lane i receives elements i, 16 + i, 32 + i, 48 + i of
 // the 64 the group addressed.  With lanes 4r ... 4r+3 on 16 consecutive columns of row k + r, lane i
-// gets column i of rows k ... k+3; two reads make the 8-element K run of a 32x32x16 operand.
+// gets column i of rows k ... k+3; two reads make the 8-element K run of an MFMA operand (32x32x16: two groups of
+// 16 lanes side by side cover a tile's 32 columns and the lane halves its two K runs; 16x16x32: one group covers the
+// tile's 16 columns and the four groups of a wave its four K runs).
 // Rows are BN * 2 bytes, a multiple of the 256 bytes the banks span, so the four rows of a read are
 // spread by XOR-ing the 64-byte unit index of a row with kmajor_swizzle_key(row).
 // ---------------------------------------------------------------------------------------------
@@ -112,8 +114,10 @@ struct RoutedGemmCfg {
   static constexpr int WTN_OUT = BN_OUT / WAVES_N;         // output columns per wave
   // The 256-row direct tiles accumulate with v_mfma_f32_16x16x32_bf16 (four accumulator registers read
   // and written per 16 K-products of a lane instead of sixteen per 16: the kernel runs at the board's
-  // power limit and the narrower accumulator traffic is worth 5 % there); the others with 32x32x16.
-  static constexpr bool MFMA16 = DIRECT_ && !B_KMAJOR_ && BM_ == 256;
+  // power limit and the narrower accumulator traffic is worth 5 % there); the others with 32x32x16.  K-major
+  // weight panels included: MaskedFFN forward + backward at d = 4096, h = 14336 runs 4.5 % (M = 4096) to 7 %
+  // (M = 32768) faster than with the backward's 256-row GEMMs on the two-stage 32x32x16 loop.
+  static constexpr bool MFMA16 = DIRECT_ && BM_ == 256;
   // Cache policy of the token panel's global->LDS loads.  The down projection's token rows (the routed intermediate,
   // read in place) pass each XCD once: a round of tiles reads a line and no later round does.  Loaded with the
   // non-temporal hint they do not push the weight panels out of L2 (cfg4 down projection 2.91 -> 2.85 ms, M = 16384
@@ -625,6 +629,11 @@ __device__ __forceinline__ void gemm_mainloop_slab_dma(const TileLanes<Cfg>& tl,
 //    (s_memtime, one lane per workgroup) put the data barrier of the two-stage form at 120 cycles per slab on
 //    the SwiGLU GEMM (K = 4096) and at 270 of 2 700 on the down projection (K = 14336), whose panels miss L2
 //    more often; the ring takes the down projection from 2.66 to 2.55 ms and leaves the SwiGLU GEMM where it was.
+//  * K-major weight panels (Cfg::B_KMAJOR, see KMajorB): the same schedule; a weight fragment is two transposing
+//    reads, issued as asm statements in the slot where the row-major form issues its one read, and every K step
+//    starts with an s_waitcnt lgkmcnt(n) that leaves outstanding only the token reads issued behind the last of
+//    them.  The range's last slab may be ragged: its surplus rows are cleared behind the data barrier that
+//    announces it (tail of the loop only).
 // =============================================================================================
 template <class Cfg>
 __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
@@ -632,8 +641,9 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
                                                       const uint32_t (&offA)[TileLanes<Cfg>::NJA],
                                                       const uint16_t* const (&baseB)[TileLanes<Cfg>::NJB],
                                                       const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
-                                                      uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN]) {
-  static_assert(Cfg::MFMA16 && Cfg::DIRECT && !Cfg::B_KMAJOR, "16x16x32 schedule of the direct 256-row tiles");
+                                                      uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN],
+                                                      const KMajorB& kb = KMajorB()) {
+  static_assert(Cfg::MFMA16 && Cfg::DIRECT, "16x16x32 schedule of the direct 256-row tiles");
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NWAVES = Cfg::NWAVES, TM = Cfg::TM, TN = Cfg::TN;
   constexpr int NJA = TileLanes<Cfg>::NJA, NJB = TileLanes<Cfg>::NJB;
@@ -644,6 +654,8 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   constexpr int RPOS = 4;                // ... ahead of the release barrier
   // Token panel in a ring of three stages: slab kt's token rows sit in stage kt % 3, its weight rows in stage kt % 2.
   constexpr bool R3 = Cfg::A_RING3;
+  constexpr bool KM = Cfg::B_KMAJOR;     // weight panel stored K-major: fragments come from transposing reads (see KMajorB)
+  constexpr int RB = Cfg::BN * 2;        // ... bytes of one of its 64 rows
   // One load per wave behind every LEV-th MFMA.  One per four MFMAs is the address unit's own rate (16 cycles per
   // load and CU).  The four-wave tiles measure faster a notch slower (SwiGLU tile 3 %, down projection 2.4 %, the
   // gathered single-weight GEMM the same either way), the eight-wave tile 1-4 % slower; six is no better than five.
@@ -668,6 +680,23 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   for (int j = 0; j < NJA; ++j) rsA[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseA[j]), 0, 0xffffffff, 0x00020000);
 #pragma unroll
   for (int j = 0; j < NJB; ++j) rsB[j] = __builtin_amdgcn_make_buffer_rsrc(wave_uniform(baseB[j]), 0, 0xffffffff, 0x00020000);
+  // K-major: one base per weight, uniform over the wave; a slab's offset goes into its resource (all scalar).
+  uint64_t kw[2] = {0, 0};
+  if constexpr (KM) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint64_t v = reinterpret_cast<uint64_t>(kb.w[i]);
+      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+      const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+      kw[i] = ((uint64_t)hi << 32) | lo;
+    }
+  }
+  auto kmajor_rsrc = [&](int kt) {
+    const int ka = kb.kt_first + kt;
+    const bool second = ka >= kb.kt_switch;
+    const uint64_t base = (second ? kw[1] : kw[0]) + (uint64_t)(uint32_t)(second ? ka - kb.kt_switch : ka) * kb.slab_bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+  };
 
   // LDS layout.  Two stages: stage s holds a slab's token panel, then its weight panel.  Ring: three token panels,
   // then two weight panels.  Token stages are named by their byte offset (a run-time value in the ring form).
@@ -681,20 +710,83 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   uint32_t b_base[TN];
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) b_base[tn] = (uint32_t)b_frag_row<Cfg>(tl.wn, tn) * kRowBytes;
+  if constexpr (KM) {
+    // This lane's 8 bytes of the first transposing read of K step 0: row 8 * lh + (i >> 2) of the slab (lh = 0..3: the
+    // lane's 8-row K run), columns 4 * (i & 3) ... of the accumulator tile's 16 (i = lane & 15); the second read of a
+    // fragment lies four rows on, the second K step 32 rows on (immediate offsets; the swizzle key repeats every 4 rows).
+    const uint32_t i = tl.lane & 15;
+    const uint32_t row = 8 * tl.lh + (i >> 2);
+    const uint32_t key = kmajor_swizzle_key<Cfg::BN>(row);
+    const uint32_t lds_addr = (uint32_t)reinterpret_cast<uintptr_t>(FFNK_LDS_PTR(lds));
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const uint32_t col = (uint32_t)b_frag_row<Cfg>(tl.wn, tn);  // first of the tile's 16 columns
+      b_base[tn] = lds_addr + row * RB + (((col / 32) ^ key) << 6) + 32 * ((col / 16) & 1) + 8 * (i & 3);
+    }
+  }
 
   zero_acc<Cfg>(acc);
   const int nk = k_len / kBK;
 
   bf16x8_t fa[TM], fb[2][TN];
+  bf16x4_t fb_lo[2][TN], fb_hi[2][TN];  // K-major: halves of a weight fragment as the two transposing reads deliver them
   auto read_a = [&](int i, int a_off, int ks) {
     fa[i] = *reinterpret_cast<const bf16x8_t*>(lds + a_off + a_base + i * 16 * kRowBytes + koff[ks]);
   };
   auto read_b = [&](int buf, int j, int b_off, int ks) {
-    fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(lds + b_off + b_base[j] + koff[ks]);
+    if constexpr (KM) {
+      // asm statements (see lds_read_tr16_b64): the compiler does not know that they are LDS reads, wait_b() stands
+      // between them and the first use
+      if (ks == 0) {
+        fb_lo[buf][j] = lds_read_tr16_b64<0>(b_base[j] + b_off);
+        fb_hi[buf][j] = lds_read_tr16_b64<4 * RB>(b_base[j] + b_off);
+      } else {
+        fb_lo[buf][j] = lds_read_tr16_b64<32 * RB>(b_base[j] + b_off);
+        fb_hi[buf][j] = lds_read_tr16_b64<36 * RB>(b_base[j] + b_off);
+      }
+    } else {
+      fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(lds + b_off + b_base[j] + koff[ks]);
+    }
+  };
+  // K-major: wait until at most `younger` LDS operations of this wave are outstanding - LDS operations return in
+  // order, so that covers every transposing read issued before the last `younger` ones - and assemble the weight
+  // fragments of buffer `buf`.  The compiler's own waits for the token fragments count only the reads it knows, i.e.
+  // they ask for no less than is needed.
+  auto wait_b = [&](int buf, auto younger) {
+    if constexpr (KM) {
+      constexpr int imm = waitcnt_imm(63, decltype(younger)::value);
+      static_assert(TN == 4 || TN == 8, "weight fragments per K step");
+      if constexpr (TN == 4)
+        asm volatile("s_waitcnt %8"
+                     : "+v"(fb_lo[buf][0]), "+v"(fb_hi[buf][0]), "+v"(fb_lo[buf][1]), "+v"(fb_hi[buf][1]), "+v"(fb_lo[buf][2]),
+                       "+v"(fb_hi[buf][2]), "+v"(fb_lo[buf][3]), "+v"(fb_hi[buf][3])
+                     : "n"(imm));
+      else
+        asm volatile("s_waitcnt %16"
+                     : "+v"(fb_lo[buf][0]), "+v"(fb_hi[buf][0]), "+v"(fb_lo[buf][1]), "+v"(fb_hi[buf][1]), "+v"(fb_lo[buf][2]),
+                       "+v"(fb_hi[buf][2]), "+v"(fb_lo[buf][3]), "+v"(fb_hi[buf][3]), "+v"(fb_lo[buf][4]), "+v"(fb_hi[buf][4]),
+                       "+v"(fb_lo[buf][5]), "+v"(fb_hi[buf][5]), "+v"(fb_lo[buf][6]), "+v"(fb_hi[buf][6]), "+v"(fb_lo[buf][7]),
+                       "+v"(fb_hi[buf][7])
+                     : "n"(imm));
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[buf][j] = __builtin_shufflevector(fb_lo[buf][j], fb_hi[buf][j], 0, 1, 2, 3, 4, 5, 6, 7);
+    }
   };
   auto load_b = [&](int l, int b_off, int kt) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(lds + b_off + (l * NWAVES + wave) * 1024), 16, offB[l],
-                                             kt * kRowBytes, 0, 0);
+    if constexpr (KM)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kmajor_rsrc(kt), FFNK_LDS_PTR(lds + b_off + (l * NWAVES + wave) * 1024), 16,
+                                               offB[l], 0, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB[l], FFNK_LDS_PTR(lds + b_off + (l * NWAVES + wave) * 1024), 16, offB[l],
+                                               kt * kRowBytes, 0, 0);
+  };
+  // K-major: clear rows [last_rows, 64) of the weight panel at b_off (the range's last slab, after it has landed and
+  // before anyone reads it).  Rows are RB contiguous bytes each, whatever the swizzle inside them.
+  auto clear_tail = [&](int b_off) {
+    uint8_t* first = lds + b_off + kb.last_rows * RB;
+    const int bytes = (kBK - kb.last_rows) * RB;
+    for (int o = (int)threadIdx.x * 16; o < bytes; o += Cfg::NT * 16) *reinterpret_cast<uint4*>(first + o) = make_uint4(0, 0, 0, 0);
+    dma_wait_barrier<0>();
   };
   auto load_a = [&](int l, int a_off, int kt) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA[l], FFNK_LDS_PTR(lds + a_off + (l * NWAVES + wave) * 1024), 16, offA[l],
@@ -726,7 +818,17 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   // following the step's first MFMAs in a row (+0.5 %).  Giving each wave its own load slot within a group of LEV
   // MFMAs (one copy of the loop per wave) or holding wave w back by 16 w cycles behind the barrier measured -0.4 %
   // and -3 %: the address unit's FIFO is not filled by the waves' coincidence.
+  // K-major: LDS reads that a step issues in slots strictly behind the slot of its last weight-fragment read (the
+  // bound wait_b() may leave outstanding at the start of the next step).
+  constexpr int G0 = BAR / TN;                        // second step: row groups ahead of the data barrier
+  constexpr int BSTEP = (NM - BAR - 2 * G0 - 2) / TN; // ... spacing of the weight-fragment reads behind it
+  static_assert(BSTEP >= 1, "no room for the weight fragments behind the barrier");
+  constexpr int kYoungerStep0 = TM - TN + 1;          // first step: the token reads of row groups TN - 1 ... TM - 1
+  constexpr int kLastB1 = BAR + 2 * G0 + (TN - 1) * BSTEP;
+  constexpr int kYoungerStep1 = TM - (kLastB1 + 1) / TN;  // second step: row groups whose last MFMA lies behind slot kLastB1
+  static_assert(kYoungerStep0 >= 0 && kYoungerStep1 >= 0 && kYoungerStep0 < 16 && kYoungerStep1 < 16, "lgkmcnt is four bits");
   auto step0 = [&](int u, int a_cur, int a_ld, int kt, bool next, bool next2) {
+    wait_b(0, std::integral_constant<int, kYoungerStep1>{});
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
@@ -746,13 +848,11 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
   // (weight stage u ^ 1, token stage at a_nxt) and loads of slab kt + 2 into the stage the release barrier freed:
   // its first L1 loads (two-stage form) or its weight panel (ring form).
   auto step1 = [&](int u, int a_nxt, int kt, bool next, bool next2) {
+    wait_b(1, std::integral_constant<int, kYoungerStep0>{});
     __builtin_amdgcn_sched_barrier(0);
     // Behind the barrier: the first-step fragments of slab kt + 1.  Token fragments of the row groups that ran
     // ahead of the barrier first, then one weight fragment every BSTEP MFMAs (the last one lands a dozen
     // MFMAs before its first use), token fragments of the other groups as their last MFMA issues.
-    constexpr int G0 = BAR / TN;                        // row groups ahead of the barrier
-    constexpr int BSTEP = (NM - BAR - 2 * G0 - 2) / TN; // spacing of the weight-fragment reads
-    static_assert(BSTEP >= 1, "no room for the weight fragments behind the barrier");
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
       if (m == RPOS) {
@@ -763,6 +863,9 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
         // slab kt + 1 has landed; the loads of slab kt + 2 issued since stay in flight
         if (next2) dma_wait_barrier<(R3 ? NJA : 0) + NPRE>();
         else dma_wait_barrier<0>();
+        if constexpr (KM) {
+          if (next && !next2 && kb.last_rows < kBK) clear_tail(b_stage(u ^ 1));  // slab kt + 1 is the last: never in the steady loop
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
       mfma(1, m);
@@ -799,6 +902,9 @@ __device__ __forceinline__ void gemm_mainloop_fixed16(const TileLanes<Cfg>& tl,
     }
   } else {
     dma_wait_barrier<0>();
+  }
+  if constexpr (KM) {
+    if (nk == 1 && kb.last_rows < kBK) clear_tail(b_stage(0));
   }
 #pragma unroll
   for (int j = 0; j < TN; ++j) read_b(0, j, b_stage(0), 0);
@@ -1075,7 +1181,7 @@ __device__ __forceinline__ void gemm_mainloop_direct(const TileLanes<Cfg>& tl,
                                                      const uint32_t (&offB)[TileLanes<Cfg>::NJB], int k_len,
                                                      uint8_t* lds, typename Cfg::Acc (&acc)[Cfg::TM][Cfg::TN],
                                                      const KMajorB& kb = KMajorB()) {
-  if constexpr (Cfg::MFMA16) gemm_mainloop_fixed16<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc);
+  if constexpr (Cfg::MFMA16) gemm_mainloop_fixed16<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
   else if constexpr (Cfg::RING) gemm_mainloop_ring<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
   else gemm_mainloop_slab_dma<Cfg>(tl, baseA, offA, baseB, offB, k_len, lds, acc, kb);
 }

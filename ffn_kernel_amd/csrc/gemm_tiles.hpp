@@ -29,8 +29,8 @@ struct PlainTiles {
 // The same tiles over K-major weights ([K, N] rows, N contiguous; direct path only).
 template <bool GATHER, bool SCATTER>
 struct KMajorTiles {
-  using T0 = RoutedGemmCfg<256, 256, 2, 4, false, GATHER, SCATTER, true, kGroupM, true>;
-  using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
+  using T0 = RoutedGemmCfg<256, 256, 2, 4, false, GATHER, SCATTER, true, kGroupM, true, kBigStagesPlain>;
+  using T1 = RoutedGemmCfg<256, 256, 2, 2, false, GATHER, SCATTER, true, kGroupM, true, kBigStagesPlain>;
   using T2 = RoutedGemmCfg<128, 128, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
   using T3 = RoutedGemmCfg<128, 64, 2, 2, false, GATHER, SCATTER, true, kGroupM, true>;
   // 128x128 behind a ring of four LDS stages, for the routed GEMMs (the weight-gradient GEMMs, whose last slab is
