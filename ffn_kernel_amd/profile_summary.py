@@ -88,6 +88,25 @@ def summarize(out: Path, workload: str, traffic_json: Path | None, min_pct: floa
             for c, v in sorted(cs.items()):
                 lines.append(f"{kernel[:100]:100s} {c:30s} n={len(v):3d} avg={sum(v) / len(v):.5g}")
                 per_kernel[(kernel, c)] = v
+    # What the counters say about each listed kernel, as far as the runs at hand allow: the clock the part held
+    # (GRBM_GUI_ACTIVE is summed over the 8 XCDs; per XCD it is the launch's duration in shader cycles, taken in another
+    # run than the traced duration), and the share of the 1024 SIMD-cycles per chip cycle in which an MFMA executed.
+    avg_ns = {r["Name"]: float(r["AverageNs"]) for r in stats} if stats else {}
+    derived = []
+    for kernel in sorted({k for (k, _) in per_kernel}):
+        def mean(c):
+            v = per_kernel.get((kernel, c))
+            return sum(v) / len(v) if v else None
+        gui, mfma = mean("GRBM_GUI_ACTIVE"), mean("SQ_VALU_MFMA_BUSY_CYCLES")
+        parts = []
+        if gui and kernel in avg_ns:
+            parts.append(f"cycles per XCD {gui / 8:.4g}, i.e. {gui / 8 / avg_ns[kernel]:.2f} GHz over the traced {avg_ns[kernel] / 1e3:.1f} us")
+        if gui and mfma:
+            parts.append(f"MFMA busy {100 * mfma / (gui / 8 * 1024):.1f} % of SIMD-cycles")
+        if parts:
+            derived.append(f"{kernel[:100]:100s} " + "; ".join(parts))
+    if derived:
+        lines += ["", "== derived per kernel =="] + derived
     cal = {}
     lines += ["", "== calibration: plain 1 GiB device copy (reads 1 GiB, writes 1 GiB per dispatch) =="]
     for counter, sub in (("FETCH_SIZE", "cfetch"), ("WRITE_SIZE", "cwrite")):
@@ -109,6 +128,9 @@ def summarize(out: Path, workload: str, traffic_json: Path | None, min_pct: floa
             lines += [f"  {k[:120]}" for k in names]
             lines.append(f"FETCH_SIZE {fetch:.5g} KiB x {cal['FETCH_SIZE']:.3f} + WRITE_SIZE {write:.5g} KiB x "
                          f"{cal['WRITE_SIZE']:.3f} = {nbytes / 1e6:.1f} MB")
+            dur = sum(avg_ns.get(k, 0.0) for k in names)
+            if dur > 0:
+                lines.append(f"over the traced {dur / 1e3:.1f} us of these kernels: {nbytes / dur:.0f} GB/s of HBM traffic")
             if traffic_json is not None:
                 table = json.loads(traffic_json.read_text()) if traffic_json.exists() else {}
                 table[workload] = {"bytes": round(nbytes), "fetch_kib": round(fetch, 1), "write_kib": round(write, 1),
