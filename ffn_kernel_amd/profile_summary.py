@@ -118,8 +118,9 @@ def summarize(out: Path, workload: str, traffic_json: Path | None, min_pct: floa
         pick = _roofline_kernels(workload)
         names = sorted({k for (k, c) in per_kernel if c == "FETCH_SIZE" and pick(k)})
         if names:
-            n_calls = min(len(per_kernel[(k, "FETCH_SIZE")]) for k in sorted({k for (k, c) in per_kernel
-                                                                                if c == "FETCH_SIZE" and _ours(k)}))
+            # calls of the workload in the run = dispatches of its most frequent kernel (a row partition shared
+            # between calls is launched once per run and weighs in with that share)
+            n_calls = max(len(per_kernel[(k, "FETCH_SIZE")]) for k in names)
             fetch = sum(sum(per_kernel[(k, "FETCH_SIZE")]) for k in names) / n_calls
             write = sum(sum(per_kernel.get((k, "WRITE_SIZE"), [0.0])) for k in names) / n_calls
             nbytes = (fetch * cal["FETCH_SIZE"] + write * cal["WRITE_SIZE"]) * 1024
