@@ -22,6 +22,7 @@ _SIGNATURES = {
     "ffnk_debug_force_tile": (c_int, [c_int]),
     "ffnk_debug_force_splits": (c_int, [c_int]),
     "ffnk_debug_force_bwd_gather": (c_int, [c_int]),
+    "ffnk_debug_force_group_m": (c_int, [c_int]),
     "ffnk_route": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "ffnk_workspace_bytes": (c_size_t, [c_int, c_int64, c_int64, c_int64]),
     "ffnk_workspace_bytes_ffn_bwd": (c_size_t, [c_int64] * 9),

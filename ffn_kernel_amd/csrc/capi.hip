@@ -73,6 +73,7 @@ RouteWs carve_route(uint8_t* ws, int64_t M) {
 // Tuner overrides, see ffnk_debug_force_tile / ffnk_debug_force_splits.
 std::atomic<int> g_force_tile{-1};    // 0..3: that tile; -1: table, then rules; -2: rules only
 std::atomic<int> g_force_splits{-1};  // >= 1: that split-K factor where a GEMM can be split
+std::atomic<int> g_force_group_m{0};      // >= 1: M-tiles per super-group in the tile order of every routed GEMM
 std::atomic<int> g_force_bwd_gather{-1};  // MaskedLinear backward: 1 = weight gradients from g and x in place, 0 = from transposes, -1 = plan
 
 int forced_tile() {
@@ -80,6 +81,11 @@ int forced_tile() {
   return (t >= 0 && t < TILE_COUNT) ? t : -1;
 }
 bool use_tuned() { return g_force_tile.load(std::memory_order_relaxed) != -2; }
+// GemmArgs::group_m of a routed GEMM: the forced value, else the measured plan's, else 0 (the tile's own).
+int plan_group_m(int op, int64_t M, int64_t k, int64_t n) {
+  if (const int f = g_force_group_m.load(std::memory_order_relaxed); f > 0) return f;
+  return use_tuned() && op != TUNED_NONE ? tuned_group_m(op, M, k, n) : 0;
+}
 int forced_splits() {
   const int s = g_force_splits.load(std::memory_order_relaxed);
   return (s >= 1 && s <= 16) ? s : -1;
@@ -453,6 +459,8 @@ int ffnk_debug_force_tile(int tile) {
   return g_force_tile.exchange(((tile >= 0 && tile < TILE_COUNT) || tile == -2) ? tile : -1);
 }
 
+int ffnk_debug_force_group_m(int group_m) { return g_force_group_m.exchange(group_m >= 1 && group_m <= 64 ? group_m : 0); }
+
 int ffnk_debug_force_bwd_gather(int on) { return g_force_bwd_gather.exchange((on == 0 || on == 1) ? on : -1); }
 
 int ffnk_debug_force_splits(int splits) { return g_force_splits.exchange((splits >= 1 && splits <= 16) ? splits : -1); }
@@ -545,7 +553,18 @@ int ffnk_tile_config(int op, int64_t M, int64_t K, int64_t N, ffnk_tile_config_t
   out->block_k = 64;
   out->waves_m = gm.waves_m;
   out->waves_n = gm.waves_n;
-  out->group_m = dual ? 8 : 4;
+  // the plan's super-group size, else the tile's own: 8 for the SwiGLU GEMM and over K-major weights (the backward's
+  // dx GEMM in the usual layout), 4 for the other single-weight GEMMs
+  int plan_gm = 0;
+  switch (op) {
+    case FFNK_OP_LINEAR_FWD: plan_gm = plan_group_m(TUNED_PLAIN, M, K, N); break;
+    case FFNK_OP_FFN_FWD:
+    case FFNK_OP_FFN_UP: plan_gm = plan_group_m(TUNED_DUAL, M, K, N); break;
+    case FFNK_OP_FFN_DOWN: plan_gm = plan_group_m(TUNED_DOWN, M, N, K); break;
+    default: plan_gm = plan_group_m(TUNED_NONE, M, K, N); break;
+  }
+  const bool kmajor_dx = op == FFNK_OP_LINEAR_BWD || op == FFNK_OP_BWD_DX;
+  out->group_m = plan_gm > 0 ? plan_gm : (dual || kmajor_dx) ? 8 : 4;
   out->split_k = splits;
   out->direct_lds = (direct || in_place) ? 1 : 0;
   out->in_place = in_place ? 1 : 0;
@@ -668,7 +687,7 @@ int ffnk_masked_linear_fwd_routed(const uint16_t* x, int64_t x_stride_m, const u
   g.B0[0] = Wv; g.B0[1] = Wt; g.B1[0] = g.B1[1] = nullptr; g.ldb = w_stride_n;
   g.C = y; g.ldc = y_stride_m;
   g.perm = rt.perm; g.counts = rt.counts;
-  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K; g.group_m = plan_group_m(TUNED_PLAIN, M, K, N);
   const bool direct = direct_ok(K, M, x_stride_m, w_stride_n);
   RoutedPlan plan = linear_plan(M, K, N);
   if (!direct) {
@@ -801,7 +820,7 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
   up.B0[0] = W1; up.B0[1] = U1; up.B1[0] = W3; up.B1[1] = U3; up.ldb = up_stride_n;
   up.C = H; up.ldc = ldh;
   up.perm = rt.perm; up.counts = rt.counts;
-  up.M = (int)M; up.N = (int)h; up.K = (int)d;
+  up.M = (int)M; up.N = (int)h; up.K = (int)d; up.group_m = plan_group_m(TUNED_DUAL, M, d, h);
   up.C_pre = pre; up.ldc_pre = pre_stride_m;
   FFNK_HIP(launch_up_gemm(routed_tile(M, h, true, d), direct_ok(d, M, x_stride_m, up_stride_n), up, stream), "up-projection GEMM");
   FFNK_HIP(mark(1), "event record");
@@ -810,7 +829,7 @@ int ffn_fwd_impl(const uint16_t* x, int64_t x_stride_m, const uint16_t* W1, cons
   dn.B0[0] = W2; dn.B0[1] = U2; dn.B1[0] = dn.B1[1] = nullptr; dn.ldb = down_stride_n;
   dn.C = out; dn.ldc = out_stride_m;
   dn.perm = rt.perm; dn.counts = rt.counts;
-  dn.M = (int)M; dn.N = (int)d; dn.K = (int)h;
+  dn.M = (int)M; dn.N = (int)d; dn.K = (int)h; dn.group_m = plan_group_m(TUNED_DOWN, M, h, d);
   const bool dn_direct = direct_ok(h, 0, ldh, down_stride_n);
   const int dn_splits = dn_direct ? tiled_down_splits(M, d, h) : 1;
   float* partials = reinterpret_cast<float*>(wsb + r.bytes + ws_align((size_t)M * ldh * 2));
@@ -952,7 +971,7 @@ int ffnk_masked_linear_bwd_routed(const uint16_t* g, int64_t g_stride_m, const u
   a.B0[0] = wt[0]; a.B0[1] = wt[1]; a.B1[0] = a.B1[1] = nullptr; a.ldb = ldw;
   a.C = dx; a.ldc = dx_stride_m;
   a.perm = rt.perm; a.counts = rt.counts;
-  a.M = (int)M; a.N = (int)K; a.K = (int)N;
+  a.M = (int)M; a.N = (int)K; a.K = (int)N; a.group_m = plan_group_m(TUNED_NONE, M, N, K);
   const int dx_tile = routed_tile(M, K, false, 0, TUNED_NONE);
   // Both GEMMs on the 128x128 tile and the weights readable in place: one launch runs the two side by
   // side (after the transposes it depends on), see below.
@@ -1051,7 +1070,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
   a.A = x; a.lda = x_stride_m;
   a.B1[0] = a.B1[1] = nullptr; a.ldb = up_stride_n;
   a.ldc = ld13; a.perm = rt.perm; a.counts = rt.counts;
-  a.M = (int)M; a.N = (int)h; a.K = (int)d;
+  a.M = (int)M; a.N = (int)h; a.K = (int)d; a.group_m = plan_group_m(TUNED_NONE, M, d, h);
   const bool up_direct = direct_ok(d, M, x_stride_m, up_stride_n);
   if (pre == nullptr) {
     a.B0[0] = W1; a.B0[1] = U1; a.C = T13;
@@ -1098,7 +1117,7 @@ int ffn_bwd_impl(const uint16_t* g, int64_t g_stride_m, const uint16_t* x, int64
     b.B0[0] = w13[0]; b.B0[1] = w13[1]; b.B1[0] = b.B1[1] = nullptr; b.ldb = ld13;
   }
   b.C = dx; b.ldc = dx_stride_m; b.perm = rt.perm; b.counts = rt.counts;
-  b.M = (int)M; b.N = (int)d; b.K = (int)(2 * h);
+  b.M = (int)M; b.N = (int)d; b.K = (int)(2 * h); b.group_m = plan_group_m(TUNED_NONE, M, 2 * h, d);
   // Few output tiles over a 2h-long contraction: split K like the forward's down projection.  The
   // fp32 partials live where the W2^T copies were (dead since the dh GEMM), if they fit there.
   const bool dx_direct = paths.dx_direct;

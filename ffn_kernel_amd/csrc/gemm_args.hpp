@@ -33,6 +33,8 @@ struct GemmArgs {
   // 3: only the remaining tiles, on the kernel's own tile, each cut into K ranges (split tail, see
   // P_tail below).
   int sched_bm = 0, sched_bn = 0, tail_mode = 0;
+  // M-tiles per super-group of the tile order (routed_tile_coord); 0 = the tile's own (RoutedGemmCfg::GROUP_M).
+  int group_m = 0;
   // Split-K (direct path, tail_mode 0, not the SwiGLU kernels): with splits > 1 the contraction is
   // cut into `splits` ranges of whole 64-element slabs, each workgroup handles one (tile, range) and
   // stores its fp32 partial sums to P[split][routed row][N]; a reduce pass adds them and scatters

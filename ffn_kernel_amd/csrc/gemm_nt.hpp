@@ -1363,7 +1363,7 @@ __device__ __forceinline__ void routed_gemm_body(const GemmArgs& g, uint8_t* lds
     }
   }
   if (L < 0) return;
-  const TileCoord tc = routed_tile_coord(L, n_vis, g.M, g.N, SBM, SBN, Cfg::GROUP_M);
+  const TileCoord tc = routed_tile_coord(L, n_vis, g.M, g.N, SBM, SBN, g.group_m > 0 ? g.group_m : Cfg::GROUP_M);
   const int grp = tc.grp;
   const int row0 = tc.row0 + sub_m * BM;  // routed position
   const int row_end = tc.row_end;

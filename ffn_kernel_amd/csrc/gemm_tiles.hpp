@@ -88,7 +88,7 @@ inline hipError_t dispatch_big_tile_with_tail(const GemmArgs& g, hipStream_t str
     a.tail_mode = 3;
     hipLaunchKernelGGL(routed_gemm_kernel<Big>, dim3(kTailSlots), dim3(Big::NT), 0, stream, a);
     if (hipError_t e = hipGetLastError()) return e;
-    return launch_routed_tail_reduce(g.P_tail, g.M, g.N, g.K, g.counts, g.perm, Big::BM, Big::BN_OUT, Big::GROUP_M, g.C,
+    return launch_routed_tail_reduce(g.P_tail, g.M, g.N, g.K, g.counts, g.perm, Big::BM, Big::BN_OUT, g.group_m > 0 ? g.group_m : Big::GROUP_M, g.C,
                                      g.ldc, stream);
   }
   a.tail_mode = 2;

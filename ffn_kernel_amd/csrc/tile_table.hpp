@@ -41,6 +41,7 @@ struct TunedPlan {
   int m_lo, m_hi;    // rows M of the call, inclusive
   int k, n;
   int tile, splits;
+  int group_m;       // M-tiles per super-group of the tile order (GemmArgs::group_m); 0 = the tile's own
 };
 }  // namespace ffnk
 #include "tile_table_gen.hpp"
@@ -50,6 +51,12 @@ inline const TunedPlan* tuned_plan(int op, int64_t M, int64_t k, int64_t n) {
   for (const TunedPlan* p = kTunedPlans; p->op >= 0; ++p)
     if (p->op == op && p->k == k && p->n == n && M >= p->m_lo && M <= p->m_hi) return p;
   return nullptr;
+}
+
+// Super-group size of a measured plan for this operation and shape, 0 where there is none (the tile's own then).
+inline int tuned_group_m(int op, int64_t M, int64_t k, int64_t n) {
+  const TunedPlan* t = tuned_plan(op, M, k, n);
+  return t ? t->group_m : 0;
 }
 
 // Routed GEMM over M rows and n_out output columns (K: the contraction, 0 = not known to the caller).

@@ -3,13 +3,17 @@ table, as the reference's find_spec searches produce its JSON tables (find_spec/
 search with min-of-3 timing; find_spec/bf16_linear_fwd.py, bf16_ffn_fwd.py, bf16_linear_bwd.py:86-99 emit
 the tables that ffn_kernel/linear.py:8-12 reads at import).
 
-The lattice is (tile id) x (split-K factor) per operation, layer shape and M bucket:
+The lattice is (tile id) x (split-K factor) x (M-tiles per super-group of the tile order) per operation, layer shape
+and M bucket - the reference's searches walk BLOCK_SIZE_M/N/K x GROUP_SIZE_M the same way (find_spec/bf16_linear_fwd.py:45-53):
   * MaskedFFN forward: the SwiGLU GEMM's tile, and the down projection's (tile, split-K factor), timed
     per stage with the events of ffnk_masked_ffn_fwd_ev;
   * MaskedLinear forward: (tile, split-K factor) of the routed GEMM, whole call;
   * MaskedLinear backward: the form of the weight-gradient GEMM (from routed transposes on the rules' tile, the same
     with both GEMMs of the fused launch behind the ring of four LDS stages, or from g and x read in place) and its
     split-K factor, whole call.
+The super-group size is searched in a second stage, from 4096 rows up (below that a call has too few M-tiles for the
+order to matter): the first stage's winner - or the rules' plan, pinned - with 2, 4, 8 and 16 M-tiles per super-group
+(ffnk_debug_force_group_m) against that plan with the tile's own size.
 Every candidate is forced through ffnk_debug_force_tile / ffnk_debug_force_splits (/ ffnk_debug_force_bwd_gather) and timed min-of-k;
 the baseline is the library's rules and cost model alone (ffnk_debug_force_tile(-2)).  The host never
 knows how many rows each group holds, and a tile's time jumps where a group's tile count crosses a
@@ -39,6 +43,8 @@ from . import _lib
 from .ops import masked_linear_backward, masked_linear_forward
 
 TILES = {0: "256x256/8w", 1: "256x256/4w", 2: "128x128/4w", 3: "small/4w", 4: "128x128/ring4"}
+GROUP_MS = (2, 4, 8, 16)   # M-tiles per super-group tried in the second stage
+GM_MIN_ROWS = 4096         # ... for buckets that reach this many rows
 TILE_IN_PLACE = 5  # weight-gradient plans only (kTileGatherDw in csrc/capi.hip): g and x read where they lie
 SPLITS = (1, 2, 3, 4, 6, 7, 8, 12, 14, 16)
 TUNED_PLAIN, TUNED_DUAL, TUNED_SPLITK, TUNED_DOWN = 0, 1, 2, 3  # TunedOp in csrc/tile_table.hpp
@@ -81,20 +87,22 @@ class _Forced:
     form goes with the tile: TILE_IN_PLACE forces it on (over the rules' tile for the dx GEMM), any other candidate
     forces it off, and the baseline (-2, -1) leaves it to the rules."""
 
-    def __init__(self, tile, splits):
-        self.tile, self.splits = tile, splits
+    def __init__(self, tile, splits, group_m=0):
+        self.tile, self.splits, self.group_m = tile, splits, group_m
 
     def __enter__(self):
         lib = _lib.load()
         lib.ffnk_debug_force_tile(-2 if self.tile == TILE_IN_PLACE else self.tile)
         lib.ffnk_debug_force_splits(self.splits)
         lib.ffnk_debug_force_bwd_gather(-1 if (self.tile, self.splits) == (-2, -1) else int(self.tile == TILE_IN_PLACE))
+        lib.ffnk_debug_force_group_m(self.group_m)
 
     def __exit__(self, *exc):
         lib = _lib.load()
         lib.ffnk_debug_force_tile(-1)
         lib.ffnk_debug_force_splits(-1)
         lib.ffnk_debug_force_bwd_gather(-1)
+        lib.ffnk_debug_force_group_m(0)
 
 
 def _ffn_stage_ms(x, W, mask, trials, ev):
@@ -180,6 +188,35 @@ def _geomean(xs):
     return p ** (1.0 / len(xs))
 
 
+def _tile_id(cfg, dual):
+    """Tile id behind an answer of ffnk_tile_config for a routed GEMM."""
+    if cfg["block_m"] == 256:
+        return 0 if cfg["waves_m"] * cfg["waves_n"] == 8 else 1
+    if cfg["lds_stages"] == 4:
+        return 4
+    return 2 if cfg["block_m"] == 128 and (dual or cfg["block_n"] == 128) else 3
+
+
+def _gm_stage(measure, ref, own, margin):
+    """Second stage: measure(g) -> [ms per scenario] (or None) of one pinned plan with g M-tiles per super-group.
+    A size is selected if, against the same plan with the tile's own size, it loses on no scenario and wins by more
+    than margin in the geometric mean - and loses on no scenario against `ref` either, the times of the plan the
+    first stage chose (or of the rules, which may pick other tiles inside the bucket than the pinned plan).
+    Returns ({g: [ms]} including the own size, selected g or None)."""
+    base = measure(own)
+    if base is None:
+        return {}, None
+    got = {own: base}
+    for g in GROUP_MS:
+        if g != own:
+            ts = measure(g)
+            if ts is not None:
+                got[g] = ts
+    cands = {g: ts for g, ts in got.items() if g != own and all(t <= r * 1.01 for t, r in zip(ts, ref))}
+    best, _ = _select(base, cands, margin)
+    return got, best
+
+
 def _select(base, cand, margin):
     """(key, geometric-mean ratio) of the best candidate measured on every scenario that loses on none and
     beats the baseline's geometric mean by more than margin; (None, 1.0) when there is none."""
@@ -236,8 +273,33 @@ def tune_ffn(d, h, bucket, trials, dev, ev, margin):
                 ups[key[0]].append(got[0])
             if key in downs:
                 downs[key].append(got[1])
+    # second stage: the super-group size, on the winner of each stage or on the rules' plan at the bucket's upper end
+    gm = {}
+    if hi >= GM_MIN_ROWS and base_cfg["up"]["path"] == _lib.PATH_MFMA_TILED:
+        best_up, _ = _select(base_up, ups, margin)
+        best_down, _ = _select(base_down, downs, margin)
+        up_plan = (best_up if best_up is not None else _tile_id(base_cfg["up"], True), 1)
+        down_plan = best_down if best_down is not None else (_tile_id(base_cfg["down"], False), base_cfg["down"]["split_k"])
+
+        def stage(plan, which):
+            def measure(g):
+                ts = []
+                for x, mask in scen:
+                    with _Forced(plan[0], plan[1], g):
+                        if which == 1 and _lib.tile_config(_lib.OP_FFN_DOWN, x.shape[0], d, h)["split_k"] != plan[1]:
+                            return None
+                        ts.append(_ffn_stage_ms(x, W, mask, trials, ev)[which])
+                return ts
+            return measure
+        up_ref = ups[best_up] if best_up is not None else base_up
+        down_ref = downs[best_down] if best_down is not None else base_down
+        got_up, g_up = _gm_stage(stage(up_plan, 0), up_ref, base_cfg["up"]["group_m"], margin)
+        got_down, g_down = _gm_stage(stage(down_plan, 1), down_ref, base_cfg["down"]["group_m"], margin)
+        gm = {"up_plan": up_plan, "up_ms": got_up, "up_group_m": g_up, "down_plan": down_plan, "down_ms": got_down,
+              "down_group_m": g_down}
     return {"op": "ffn_fwd", "d": d, "h": h, "m_lo": lo, "m_hi": hi, "rules": base_cfg, "rules_up_ms": base_up,
-            "rules_down_ms": base_down, "up_first_ms": ups0, "down_first_ms": downs0, "up_ms": ups, "down_ms": downs}
+            "rules_down_ms": base_down, "up_first_ms": ups0, "down_first_ms": downs0, "up_ms": ups, "down_ms": downs,
+            "group_m": gm}
 
 
 def _tune_call(make_fn, scen_inputs, candidates, trials, margin):
@@ -283,8 +345,23 @@ def tune_linear_fwd(K, N, bucket, trials, dev, margin):
                               lambda M, s=s: _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, N)["split_k"] == s))
     base, first, full = _tune_call(lambda inp: (lambda: masked_linear_forward(inp[0], Wv.T, Wt.T, inp[1])),
                                    scen, cands, trials, margin)
+    gm = {}
+    if hi >= GM_MIN_ROWS and base_cfg["path"] == _lib.PATH_MFMA_TILED:
+        best, _ = _select(base, full, margin)
+        plan = best if best is not None else (_tile_id(base_cfg, False), base_cfg["split_k"])
+
+        def measure(g):
+            ts = []
+            for x, mask in scen:
+                with _Forced(plan[0], plan[1], g):
+                    if _lib.tile_config(_lib.OP_LINEAR_FWD, x.shape[0], K, N)["split_k"] != plan[1]:
+                        return None
+                    ts.append(_call_ms(lambda: masked_linear_forward(x, Wv.T, Wt.T, mask), trials))
+            return ts
+        got, g_sel = _gm_stage(measure, full[best] if best is not None else base, base_cfg["group_m"], margin)
+        gm = {"plan": plan, "ms": got, "group_m": g_sel}
     return {"op": "linear_fwd", "K": K, "N": N, "m_lo": lo, "m_hi": hi, "rules": base_cfg, "rules_ms": base,
-            "first_ms": first, "ms": full}
+            "first_ms": first, "ms": full, "group_m": gm}
 
 
 def tune_linear_bwd(K, N, bucket, trials, dev, margin):
@@ -307,28 +384,33 @@ def tune_linear_bwd(K, N, bucket, trials, dev, margin):
 
 
 def plans_from(records, margin):
-    """Table entries (op, m_lo, m_hi, k, n, tile, splits) for every record with a candidate that loses on
-    no scenario and beats the rules' geometric-mean time by more than `margin`."""
+    """Table entries (op, m_lo, m_hi, k, n, tile, splits, group_m) for every record with a candidate that loses on
+    no scenario and beats the rules' geometric-mean time by more than `margin`; a super-group size that won the second
+    stage comes with the plan it was measured on (the first stage's winner, or the rules' plan pinned)."""
     out = []
     for r in records:
+        gm = r.get("group_m") or {}
         if r["op"] == "ffn_fwd":
             tile, _ = _select(r["rules_up_ms"], r["up_ms"], margin)
-            if tile is not None:
-                out.append((TUNED_DUAL, r["m_lo"], r["m_hi"], r["d"], r["h"], tile, 1))
+            if tile is not None or gm.get("up_group_m"):
+                plan = gm["up_plan"] if gm.get("up_group_m") else (tile, 1)
+                out.append((TUNED_DUAL, r["m_lo"], r["m_hi"], r["d"], r["h"], plan[0], 1, gm.get("up_group_m") or 0))
             key, _ = _select(r["rules_down_ms"], r["down_ms"], margin)
-            if key is not None:
-                out.append((TUNED_DOWN, r["m_lo"], r["m_hi"], r["h"], r["d"], key[0], key[1]))
+            if key is not None or gm.get("down_group_m"):
+                plan = gm["down_plan"] if gm.get("down_group_m") else key
+                out.append((TUNED_DOWN, r["m_lo"], r["m_hi"], r["h"], r["d"], plan[0], plan[1], gm.get("down_group_m") or 0))
         elif r["op"] == "linear_fwd":
             key, _ = _select(r["rules_ms"], r["ms"], margin)
-            if key is not None:
-                out.append((TUNED_PLAIN, r["m_lo"], r["m_hi"], r["K"], r["N"], key[0], key[1]))
+            if key is not None or gm.get("group_m"):
+                plan = gm["plan"] if gm.get("group_m") else key
+                out.append((TUNED_PLAIN, r["m_lo"], r["m_hi"], r["K"], r["N"], plan[0], plan[1], gm.get("group_m") or 0))
         elif r["op"] == "linear_bwd":
             key, _ = _select(r["rules_ms"], r["ms"], margin)
             if key is not None:
                 tile, s = key
                 if tile < 0:
                     tile = {(256, 256): 0, (128, 128): 2}.get((r["rules_xpose"]["block_m"], r["rules_xpose"]["block_n"]), 2)
-                out.append((TUNED_SPLITK, r["m_lo"], r["m_hi"], r["N"], r["K"], tile, s))  # R = N, Cc = K (dW stored [N, K])
+                out.append((TUNED_SPLITK, r["m_lo"], r["m_hi"], r["N"], r["K"], tile, s, 0))  # R = N, Cc = K (dW stored [N, K])
     # one entry per key (the operation is part of it: a linear layer and an FFN's down projection of the
     # same extents are different kernels and keep their own plans)
     seen, uniq = set(), []
@@ -341,11 +423,11 @@ def plans_from(records, margin):
 
 def render_header(plans) -> str:
     lines = ["// Measured plans of the gfx950 tile table.  GENERATED by `python -m ffn_kernel_amd.tune --emit`: do not edit.",
-             "// {op, m_lo, m_hi, k, n, tile, splits}; see TunedPlan in tile_table.hpp.",
+             "// {op, m_lo, m_hi, k, n, tile, splits, group_m}; see TunedPlan in tile_table.hpp.",
              "#pragma once", "namespace ffnk {", "constexpr TunedPlan kTunedPlans[] = {"]
     for e in plans:
-        lines.append("    {%d, %d, %d, %d, %d, %d, %d}," % e)
-    lines += ["    {-1, 0, 0, 0, 0, 0, 0},", "};", "}  // namespace ffnk", ""]
+        lines.append("    {%d, %d, %d, %d, %d, %d, %d, %d}," % e)
+    lines += ["    {-1, 0, 0, 0, 0, 0, 0, 0},", "};", "}  // namespace ffnk", ""]
     return "\n".join(lines)
 
 
@@ -353,7 +435,7 @@ def read_header(path) -> list:
     """The entries of a generated header (the terminator excluded), as render_header wrote them."""
     import re
     out = []
-    for m in re.finditer(r"^\s*\{(-?\d+(?:,\s*-?\d+){6})\},", Path(path).read_text(), re.M):
+    for m in re.finditer(r"^\s*\{(-?\d+(?:,\s*-?\d+){7})\},", Path(path).read_text(), re.M):
         e = tuple(int(v) for v in m.group(1).split(","))
         if e[0] >= 0:
             out.append(e)
@@ -414,6 +496,19 @@ def main(argv=None) -> int:
     def ratios(base, cand):
         return "  ".join(f"{k}:" + "/".join(f"{t / b_:.2f}" for t, b_ in zip(ts, base)) for k, ts in cand.items()) or "-"
 
+    def gm_text(r):
+        """Second stage of a record: per stage, the pinned plan (tile, splits), the tile's own super-group size, and
+        group_m:time / the plan's time with its own size, per scenario."""
+        gm = r.get("group_m") or {}
+        parts = []
+        for stage, plan, ms in (("up ", "up_plan", "up_ms"), ("down ", "down_plan", "down_ms"), ("", "plan", "ms")):
+            if plan not in gm or not gm[ms]:
+                continue
+            own = r["rules"][stage.strip()]["group_m"] if stage else r["rules"]["group_m"]
+            others = {g: ts for g, ts in gm[ms].items() if g != own}
+            parts.append(f"{stage}group_m on {tuple(gm[plan])} (own {own}): {ratios(gm[ms][own], others)}")
+        return (" | " + " ; ".join(parts)) if parts else ""
+
     for d, h in (ffn_layers if "ffn_fwd" in ops else []):
         for b in buckets:
             if b[1] * h * 2 > 4 << 30:
@@ -424,14 +519,14 @@ def main(argv=None) -> int:
             print(f"ffn_fwd    d={d:5d} h={h:5d} M<={b[1]:6d} | rules up {_fmt_list(r['rules_up_ms'])} "
                   f"(tile {up['block_m']}x{up['block_n']}/{up['waves_m'] * up['waves_n']}w) down {_fmt_list(r['rules_down_ms'])}"
                   f" | up tile:ratio per scenario {ratios(r['rules_up_ms'], r['up_ms'])}"
-                  f" | down (tile, splits):ratio {ratios(r['rules_down_ms'], r['down_ms'])}", flush=True)
+                  f" | down (tile, splits):ratio {ratios(r['rules_down_ms'], r['down_ms'])}" + gm_text(r), flush=True)
     for K, N in linear_layers:
         for b in buckets:
             if "linear_fwd" in ops:
                 r = tune_linear_fwd(K, N, b, args.trials, dev, args.margin)
                 records.append(r)
                 print(f"linear_fwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} | (tile, splits):ratio "
-                      f"{ratios(r['rules_ms'], r['ms'])}", flush=True)
+                      f"{ratios(r['rules_ms'], r['ms'])}" + gm_text(r), flush=True)
             if "linear_bwd" in ops:
                 r = tune_linear_bwd(K, N, b, args.trials, dev, args.margin)
                 records.append(r)
@@ -446,7 +541,7 @@ def main(argv=None) -> int:
         plans = sorted(plans + kept)
     print(f"{len(plans)} measured plans lose on no scenario and beat the rules by more than {args.margin:.0%}:")
     for e in plans:
-        print("   op=%d M in [%d, %d] k=%d n=%d -> tile %d, splits %d" % e)
+        print("   op=%d M in [%d, %d] k=%d n=%d -> tile %d, splits %d, group_m %d" % e)
     if args.json:
         def keyed(d):
             return {str(k): v for k, v in d.items()} if isinstance(d, dict) else d

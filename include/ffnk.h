@@ -145,6 +145,11 @@ FFNK_API int ffnk_debug_force_splits(int splits);
  * (rows found through perm) wherever the operands allow it, 0 = it reads routed, padded transposes written by an
  * elementwise pass first, -1 = the plan decides.  Returns the previous value. */
 FFNK_API int ffnk_debug_force_bwd_gather(int on);
+/* Tuner-only as well: every routed GEMM walks its tiles in super-groups of `group_m` M-tiles (1..64) instead of the
+ * tile's own (8 for the SwiGLU GEMM and the K-major kernels, 4 for the other single-weight GEMMs); 0 returns to those.
+ * The counterpart of the GROUP_SIZE_M dimension of the reference's searches (find_spec/bf16_linear_fwd.py:45-53).
+ * Returns the previous value. */
+FFNK_API int ffnk_debug_force_group_m(int group_m);
 
 /*
  * MaskedLinear forward — replaces _bf16_linear_forward (ffn_kernel/linear.py:418-452):

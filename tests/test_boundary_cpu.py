@@ -116,10 +116,19 @@ def test_tile_table_entries():
         assert _lib.tile_config(_lib.OP_BWD_DW, 8192, 1024, 1024)["in_place"] == 0
         lib.ffnk_debug_force_bwd_gather(1)
         assert _lib.tile_config(_lib.OP_BWD_DW, 8192, 4096, 4096)["in_place"] == 1
+        # M-tiles per super-group of the tile order: the tile's own unless a plan or the hook says otherwise
+        assert _lib.tile_config(_lib.OP_FFN_UP, 32768, 4096, 14336)["group_m"] == 8
+        assert _lib.tile_config(_lib.OP_FFN_DOWN, 32768, 4096, 14336)["group_m"] == 4
+        assert _lib.tile_config(_lib.OP_BWD_DX, 32768, 4096, 4096)["group_m"] == 8   # K-major weights
+        assert lib.ffnk_debug_force_group_m(2) == 0
+        assert _lib.tile_config(_lib.OP_FFN_UP, 32768, 4096, 14336)["group_m"] == 2
+        assert _lib.tile_config(_lib.OP_LINEAR_FWD, 32768, 4096, 4096)["group_m"] == 2
+        assert lib.ffnk_debug_force_group_m(1000) == 2 and lib.ffnk_debug_force_group_m(0) == 0   # out of range: back to the plans
     finally:
         lib.ffnk_debug_force_splits(-1)
         lib.ffnk_debug_force_tile(-1)
         lib.ffnk_debug_force_bwd_gather(-1)
+        lib.ffnk_debug_force_group_m(0)
     with pytest.raises(ValueError):
         _lib.tile_config(77, 1, 1, 1)
 
@@ -226,7 +235,7 @@ def test_measured_plans_are_consulted_before_the_rules():
     file byte for byte from its own entries."""
     from ffn_kernel_amd import tune
     text = tune.GEN_PATH.read_text()
-    entries = [tuple(map(int, e)) for e in re.findall(r"^\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},$", text, re.M)]
+    entries = [tuple(map(int, e)) for e in re.findall(r"^\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},$", text, re.M)]
     assert tune.render_header(entries) == text
     # what `--ops` keeps of a table it re-measures only in part is read back with the tuner's own parser
     assert tune.read_header(tune.GEN_PATH) == entries
@@ -234,11 +243,13 @@ def test_measured_plans_are_consulted_before_the_rules():
     geom = {0: (256, 256, 8), 1: (256, 256, 4), 2: (128, 128, 4), 4: (128, 128, 4)}
     lib = _lib.load()
     checked = 0
-    for op, lo, hi, k, n, tile, splits in entries:
+    for op, lo, hi, k, n, tile, splits, group_m in entries:
+        assert group_m in (0, 2, 4, 8, 16) and (group_m == 0 or op != tune.TUNED_SPLITK)
         if op == tune.TUNED_DUAL:
             cfg = _lib.tile_config(_lib.OP_FFN_UP, hi, k, n)
             if tile in geom:
                 assert (cfg["block_m"], cfg["waves_m"] * cfg["waves_n"]) == (geom[tile][0], geom[tile][2]), (op, hi, k, n, cfg)
+            assert cfg["group_m"] == (group_m or 8), (op, hi, k, n, cfg)  # the plan's super-group size, else the SwiGLU tiles' own
             checked += 1
         elif op == tune.TUNED_PLAIN:
             cfg = _lib.tile_config(_lib.OP_LINEAR_FWD, hi, k, n)
@@ -279,7 +290,7 @@ def test_measured_plans_are_consulted_before_the_rules():
     ops_seen = {e[0] for e in entries}
     assert ops_seen <= {tune.TUNED_PLAIN, tune.TUNED_DUAL, tune.TUNED_SPLITK, tune.TUNED_DOWN}
     if entries:
-        op, lo, hi, k, n, tile, splits = next((e for e in entries if e[0] == tune.TUNED_DOWN), entries[0])
+        op, lo, hi, k, n, tile, splits, _ = next((e for e in entries if e[0] == tune.TUNED_DOWN), entries[0])
         try:
             assert lib.ffnk_debug_force_tile(-2) == -1
             rules = _lib.tile_config(_lib.OP_FFN_DOWN, hi, n, k)

@@ -880,6 +880,32 @@ def test_linear_bwd_fused_launch(dev, M, K, N, p):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("group_m", [1, 2, 16])
+def test_forced_super_group_size(dev, group_m):
+    """The tile order is a permutation of the same tiles for every super-group size (ffnk_debug_force_group_m), also
+    where the launch is cut into whole rounds and a remainder: MaskedLinear and MaskedFFN forward against the oracle
+    on shapes with more than 256 tiles of 256 rows, and the reduce pass of a split tail walks the same order."""
+    note(f"forced group_m={group_m}")
+    lib = _lib.load()
+    M, K, N = 8300, 128, 2304
+    mask = torch.rand(M, generator=torch.Generator().manual_seed(11)) < 0.45
+    wlin = wl.make_linear("t", M, K, N, mask, seed=12, w_std=0.05)
+    wffn = wl.make_ffn("t", M, 128, 1152, mask, seed=13, w_std=0.05)
+    dl, df = wlin.to(dev), wffn.to(dev)
+    try:
+        lib.ffnk_debug_force_group_m(group_m)
+        lib.ffnk_debug_force_tile(0)
+        assert _lib.tile_config(_lib.OP_LINEAR_FWD, M, K, N)["group_m"] == group_m
+        y = MaskedLinear.apply(dl.x, dl.Wv.T, dl.Wt.T, dl.mask)
+        out = MaskedFFN.apply(df.x, *[df.W[k].T for k in ("w1", "w2", "w3", "u1", "u2", "u3")], df.mask)
+        torch.cuda.synchronize()
+    finally:
+        lib.ffnk_debug_force_group_m(0)
+        lib.ffnk_debug_force_tile(-1)
+    assert_close(y, cref.linear_fwd(wlin.x, wlin.Wv, wlin.Wt, wlin.mask), "linear fwd")
+    assert_close(out, cref.ffn_fwd(wffn.x, wffn.W, wffn.mask, round_mid=True), "ffn fwd")
+
+
 @pytest.fixture
 def force_bwd_form():
     """ffnk_debug_force_bwd_gather / ffnk_debug_force_splits for one test; back to the plans afterwards."""

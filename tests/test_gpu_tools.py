@@ -41,15 +41,17 @@ def test_tuner_emits_a_table_the_library_can_compile(dev, tmp_path, capsys):
     out = tmp_path / "tile_table_gen.hpp"
     assert tune.main(["--quick", "--trials", "2", "--emit", "--out", str(out), "--json", str(tmp_path / "t.json")]) == 0
     text = out.read_text()
-    entries = re.findall(r"^\s*\{(-?\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},$", text, re.M)
+    entries = re.findall(r"^\s*\{(-?\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\},$", text, re.M)
     assert entries and entries[-1][0] == "-1"
-    for op, lo, hi, k, n, tile, splits in entries[:-1]:
+    for op, lo, hi, k, n, tile, splits, group_m in entries[:-1]:
+        assert int(group_m) in (0, 2, 4, 8, 16)
         # tile 5 is a form of the weight-gradient GEMM (operands read in place), not a tile of the routed GEMMs
         assert int(op) in (0, 1, 2, 3) and int(lo) <= int(hi) and 0 <= int(tile) <= (5 if int(op) == 2 else 4) and 1 <= int(splits) <= 16
     recs = json.loads((tmp_path / "t.json").read_text())
     assert {r["op"] for r in recs} == {"ffn_fwd", "linear_fwd", "linear_bwd"}
     lib = _lib.load()
     assert lib.ffnk_debug_force_tile(-1) == -1 and lib.ffnk_debug_force_splits(-1) == -1 and lib.ffnk_debug_force_bwd_gather(-1) == -1
+    assert lib.ffnk_debug_force_group_m(0) == 0
 
 
 def test_forced_splits_results_match(dev):
