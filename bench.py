@@ -2,8 +2,10 @@
 MI355X (BASELINE.json's metric, `configs[3]`).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload cfg4|cfg2|cfg1|cfg3|decode1v|decode1t|decode8|decode32|decode64|decode64v|prefill1024]
+                    [--workload cfg4|cfg2|cfg1|cfg3|decode1v|decode1t|decode8|decode32|decode64|decode64v|prefillN]
                     [--no-route-cache]
+                    [--workload gemm_ref|gemm_ref_down|copy1g]   (reference points, not this library: the vendor
+                     library's plain GEMM on the up / down projection's shape; the 1 GiB copy that calibrates counters)
 
 A step is one pass of the hot path over the whole synthetic batch, inputs already resident in HBM:
   cfg4 / cfg2 / decodeN / prefillN : one MaskedFFN.apply (row partition + up-projection with SwiGLU +
