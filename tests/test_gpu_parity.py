@@ -971,6 +971,44 @@ def test_linear_bwd_weight_gradients_in_place_and_from_transposes(dev, force_bwd
         assert torch.equal(a, b)
 
 
+def test_linear_bwd_forms_on_random_shapes(dev, force_bwd_form):
+    """Both forms of the weight-gradient GEMM on 24 seeded random shapes (single rows, groups shorter than a slab,
+    K and N below a tile, padded row strides, masks from all-text to all-visual) against the row-select form in
+    double precision computed with torch on the GPU."""
+    gen = torch.Generator().manual_seed(2024)
+
+    def rnd(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=gen))
+    for case in range(24):
+        M = (1, 2, 63, 65)[case] if case < 4 else rnd(3, 3000)
+        K, N = 8 * rnd(1, 65), 8 * rnd(1, 65)
+        p = (0.0, 1.0, 0.5, 0.02, 0.98)[case % 5]
+        pad_g, pad_x = 8 * rnd(0, 2), 8 * rnd(0, 2)
+        note(f"linear bwd random case {case}: M={M} K={K} N={N} p={p} pads {pad_g} {pad_x}")
+        mask = (torch.rand(M, generator=gen) < p).to(dev)
+        gw_ = (torch.randn(M, N + pad_g, generator=gen)).to(torch.bfloat16).to(dev)
+        xw_ = (torch.randn(M, K + pad_x, generator=gen)).to(torch.bfloat16).to(dev)
+        g, x = gw_[:, :N], xw_[:, :K]
+        Wv = (torch.randn(N, K, generator=gen) * 0.05).to(torch.bfloat16).to(dev)
+        Wt = (torch.randn(N, K, generator=gen) * 0.05).to(torch.bfloat16).to(dev)
+        gd, xd = g.double(), x.double()
+        mv = mask.double()[:, None]
+        ref_dx = torch.where(mask[:, None], gd @ Wv.double(), gd @ Wt.double()).cpu()
+        ref_dwv = ((gd * mv).T @ xd).cpu()          # [N, K]
+        ref_dwt = ((gd * (1 - mv)).T @ xd).cpu()
+        for in_place in (0, 1):
+            force_bwd_form(in_place, -1)
+            dx, dbv, dbt = masked_linear_backward(g, x, Wv.T, Wt.T, mask)
+            force_bwd_form(-1, -1)
+            assert_close(dx, ref_dx, f"case {case} form {in_place} dx")
+            assert_close(dbv.T, ref_dwv, f"case {case} form {in_place} dWv")
+            assert_close(dbt.T, ref_dwt, f"case {case} form {in_place} dWt")
+            if not bool(mask.any()):
+                assert torch.count_nonzero(dbv) == 0
+            if bool(mask.all()):
+                assert torch.count_nonzero(dbt) == 0
+
+
 @pytest.mark.parametrize("in_place", [0, 1])
 def test_linear_bwd_non_finite_rows_stay_in_their_modality(dev, force_bwd_form, in_place):
     """Inf / NaN in the text rows of g and x reach dW_t only: the visual gradient is what it is without them, also
