@@ -792,7 +792,9 @@ def test_forced_tile_linear_fwd_bwd(dev, force_tile, tile, M, K, N, p):
 
 
 @pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
-@pytest.mark.parametrize("M,d,h,p", [(700, 256, 512, 0.5), (300, 128, 320, 0.4)])
+@pytest.mark.parametrize("M,d,h,p", [(700, 256, 512, 0.5), (300, 128, 320, 0.4),
+                                     (70, 128, 192, 0.5),     # one ragged slab of contraction rows per modality
+                                     (180, 192, 256, 0.45)])  # two, the second ragged
 def test_forced_tile_ffn_fwd_bwd(dev, force_tile, tile, M, d, h, p):
     note(f"forced tile {tile}: ffn fwd+bwd M={M} d={d} h={h}")
     gen = torch.Generator().manual_seed(M + tile)
