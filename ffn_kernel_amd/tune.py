@@ -26,6 +26,7 @@ geometric-mean time beats the baseline by more than --margin.
 
     python -m ffn_kernel_amd.tune                 # sweep, print the comparison
     python -m ffn_kernel_amd.tune --emit          # ... and rewrite csrc/tile_table_gen.hpp (then rebuild)
+    python -m ffn_kernel_amd.tune --passes 2 --emit   # two sweeps; a plan must win in both (the committed table)
     python -m ffn_kernel_amd.tune --quick         # two buckets per layer (smoke test of the harness)
     python -m ffn_kernel_amd.tune --ffn 5120,13824 --linear 5120,5120 --emit   # ... with a model's own layers added
 """
@@ -462,6 +463,9 @@ def main(argv=None) -> int:
                     help="MaskedFFN layer to measure besides the default ones (repeatable)")
     ap.add_argument("--linear", action="append", default=None, metavar="K,N",
                     help="MaskedLinear layer to measure besides the default ones (repeatable)")
+    ap.add_argument("--passes", type=int, default=1,
+                    help="independent sweeps; only a plan that every one of them selects enters the table (timing "
+                         "noise makes plans near the margin come and go between sweeps)")
     ap.add_argument("--ops", default=",".join(OPS), help="operations to measure (comma separated); --emit keeps the "
                     f"plans that {GEN_PATH.name} holds for the others")
     args = ap.parse_args(argv)
@@ -491,7 +495,6 @@ def main(argv=None) -> int:
     torch.cuda.set_device(dev)
     ev = _Events()
     buckets = [BUCKETS[1], BUCKETS[4]] if args.quick else BUCKETS
-    records = []
 
     def ratios(base, cand):
         return "  ".join(f"{k}:" + "/".join(f"{t / b_:.2f}" for t, b_ in zip(ts, base)) for k, ts in cand.items()) or "-"
@@ -509,31 +512,39 @@ def main(argv=None) -> int:
             parts.append(f"{stage}group_m on {tuple(gm[plan])} (own {own}): {ratios(gm[ms][own], others)}")
         return (" | " + " ; ".join(parts)) if parts else ""
 
-    for d, h in (ffn_layers if "ffn_fwd" in ops else []):
-        for b in buckets:
-            if b[1] * h * 2 > 4 << 30:
-                continue
-            r = tune_ffn(d, h, b, args.trials, dev, ev, args.margin)
-            records.append(r)
-            up = r["rules"]["up"]
-            print(f"ffn_fwd    d={d:5d} h={h:5d} M<={b[1]:6d} | rules up {_fmt_list(r['rules_up_ms'])} "
-                  f"(tile {up['block_m']}x{up['block_n']}/{up['waves_m'] * up['waves_n']}w) down {_fmt_list(r['rules_down_ms'])}"
-                  f" | up tile:ratio per scenario {ratios(r['rules_up_ms'], r['up_ms'])}"
-                  f" | down (tile, splits):ratio {ratios(r['rules_down_ms'], r['down_ms'])}" + gm_text(r), flush=True)
-    for K, N in linear_layers:
-        for b in buckets:
-            if "linear_fwd" in ops:
-                r = tune_linear_fwd(K, N, b, args.trials, dev, args.margin)
+    per_pass = []
+    for pass_no in range(max(1, args.passes)):
+        if args.passes > 1:
+            print(f"== sweep {pass_no + 1} of {args.passes} ==", flush=True)
+        records = []
+        for d, h in (ffn_layers if "ffn_fwd" in ops else []):
+            for b in buckets:
+                if b[1] * h * 2 > 4 << 30:
+                    continue
+                r = tune_ffn(d, h, b, args.trials, dev, ev, args.margin)
                 records.append(r)
-                print(f"linear_fwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} | (tile, splits):ratio "
-                      f"{ratios(r['rules_ms'], r['ms'])}" + gm_text(r), flush=True)
-            if "linear_bwd" in ops:
-                r = tune_linear_bwd(K, N, b, args.trials, dev, args.margin)
-                records.append(r)
-                print(f"linear_bwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} (splits {r['rules']['split_k']}"
-                      f"{', in place' if r['rules']['in_place'] else ''}) | (tile, splits):ratio {ratios(r['rules_ms'], r['ms'])}",
-                      flush=True)
-    plans = plans_from(records, args.margin)
+                up = r["rules"]["up"]
+                print(f"ffn_fwd    d={d:5d} h={h:5d} M<={b[1]:6d} | rules up {_fmt_list(r['rules_up_ms'])} "
+                      f"(tile {up['block_m']}x{up['block_n']}/{up['waves_m'] * up['waves_n']}w) down {_fmt_list(r['rules_down_ms'])}"
+                      f" | up tile:ratio per scenario {ratios(r['rules_up_ms'], r['up_ms'])}"
+                      f" | down (tile, splits):ratio {ratios(r['rules_down_ms'], r['down_ms'])}" + gm_text(r), flush=True)
+        for K, N in linear_layers:
+            for b in buckets:
+                if "linear_fwd" in ops:
+                    r = tune_linear_fwd(K, N, b, args.trials, dev, args.margin)
+                    records.append(r)
+                    print(f"linear_fwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} | (tile, splits):ratio "
+                          f"{ratios(r['rules_ms'], r['ms'])}" + gm_text(r), flush=True)
+                if "linear_bwd" in ops:
+                    r = tune_linear_bwd(K, N, b, args.trials, dev, args.margin)
+                    records.append(r)
+                    print(f"linear_bwd K={K:5d} N={N:5d} M<={b[1]:6d} | rules {_fmt_list(r['rules_ms'])} (splits {r['rules']['split_k']}"
+                          f"{', in place' if r['rules']['in_place'] else ''}) | (tile, splits):ratio {ratios(r['rules_ms'], r['ms'])}",
+                          flush=True)
+        per_pass.append(plans_from(records, args.margin))
+    plans = [e for e in per_pass[0] if all(e in other for other in per_pass[1:])]
+    if args.passes > 1:
+        print(f"plans per sweep: {[len(p_) for p_ in per_pass]}; selected by every sweep: {len(plans)}")
     if len(ops) < len(OPS):
         measured = {k for o in ops for k in OP_KINDS[o]}
         kept = [e for e in read_header(GEN_PATH) if e[0] not in measured]
